@@ -1,0 +1,224 @@
+/*
+ * rgd_hip.h -- C ABI of librgd_hip.so: gfx950 (MI355X) HIP kernels for the rgd-triton operator set.
+ *
+ * Each entry point replaces one host launch wrapper of the reference (the function that sits
+ * between a torch.autograd.Function and its @triton.jit kernels); the reference file:line is
+ * given with every declaration (paths relative to the reference checkout, rgd_triton/triton/...).
+ *
+ * Conventions
+ *   - plain pointers and sizes only; every pointer is a DEVICE pointer owned by the caller.
+ *     The library never allocates or frees device memory.
+ *   - strides are in ELEMENTS (not bytes) and may be any value that keeps accesses in bounds;
+ *     the last dimension of every tensor is unit stride.  A stride of 0 broadcasts.
+ *   - dtype codes: RGD_F32 / RGD_F16 / RGD_BF16.  All statistics and accumulation are fp32.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Calls only enqueue
+ *     work and return; they never synchronise.
+ *   - return value 0 on success, negative rgd_status otherwise; rgd_last_error() returns a
+ *     thread-local message for the last failure on the calling thread.
+ *   - functions are re-entrant; the only state is the loaded code object.
+ */
+#ifndef RGD_HIP_H
+#define RGD_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum rgd_dtype { RGD_F32 = 0, RGD_F16 = 1, RGD_BF16 = 2 };
+
+enum rgd_status {
+    RGD_OK = 0,
+    RGD_ERR_INVALID = -1,     /* bad argument (shape, dtype code, null pointer)          */
+    RGD_ERR_UNSUPPORTED = -2, /* valid but outside what the kernels cover                 */
+    RGD_ERR_LAUNCH = -3,      /* hipLaunchKernel reported an error                        */
+    RGD_ERR_WORKSPACE = -4    /* caller-provided workspace too small                      */
+};
+
+enum rgd_bias_kind { RGD_BIAS_NONE = 0, RGD_BIAS_VECTOR = 1, RGD_BIAS_MATRIX = 2 };
+
+/* (B, T, C) tensor of rows; element (b, n, c) lives at ptr + b*stride_b + n*stride_n + c.
+ * For a weight (B,1,C) only stride_b is used (0 = one weight shared by the batch). */
+typedef struct rgd_tensor3 {
+    void*   ptr;
+    int64_t stride_b;
+    int64_t stride_n;
+} rgd_tensor3;
+
+/* (B, H, T, D) tensor addressed by (batch, head, token) strides whatever its memory order:
+ * heads_second=True passes (stride(0), stride(1), stride(2)), heads_second=False passes
+ * (stride(0), stride(2), stride(1)) -- the reference resolves layouts the same way
+ * (normalization/head_layernorm_cached.py:216-231). */
+typedef struct rgd_tensor4 {
+    void*   ptr;
+    int64_t stride_b;
+    int64_t stride_h;
+    int64_t stride_n;
+} rgd_tensor4;
+
+/* library / ABI version (major*1000 + minor) and last error text */
+int         rgd_version(void);
+const char* rgd_last_error(void);
+
+/* ------------------------------------------------------------------------------------------
+ * RMSNorm  y = x * rsqrt(mean(x^2) + eps) * w        x (B,T,C), w (B,1,C) or shared
+ * ------------------------------------------------------------------------------------------ */
+
+/* replaces _rms_fwd, normalization/rmsnorm_cached.py:319-403 (kernel :6-103) */
+int rgd_rms_fwd(int64_t B, int64_t T, int64_t C,
+                const rgd_tensor3* x, const rgd_tensor3* w, const rgd_tensor3* y,
+                int x_dtype, int w_dtype, float eps, void* stream);
+
+/* Scratch the backward needs for the deterministic dw reduction.
+ * *workspace_bytes: size of `workspace` (any contents on entry).
+ * *counter_bytes:   size of `counters`; MUST be zero-filled before the first call that uses the
+ *                   buffer; every call leaves it zero-filled again, so it can be reused by
+ *                   successive calls on one stream without clearing.  Calls that may overlap
+ *                   (different streams) need separate counter and workspace buffers. */
+int rgd_rms_bwd_workspace(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2,
+                          size_t* workspace_bytes, size_t* counter_bytes);
+
+/* replaces _rms_bwd, normalization/rmsnorm_cached.py:406-569 (kernels :106-264 and :269-313):
+ *   dx = (dy*w - xhat*mean(xhat*dy*w)) * rrms,   dw[b or shared] = sum_rows xhat*dy.
+ * dw is (B,1,C) addressed with dw->stride_b when w_shared == 0, and a single (C) row holding the
+ * sum over the batch when w_shared != 0 (the reference sums a (B,1,C) buffer on the host,
+ * rmsnorm_cached.py:623-625).  dw is accumulated in fp32, in a fixed order, and stored in w_dtype. */
+int rgd_rms_bwd(int64_t B, int64_t T, int64_t C,
+                const rgd_tensor3* dy, const rgd_tensor3* x, const rgd_tensor3* w,
+                const rgd_tensor3* dx, const rgd_tensor3* dw, int w_shared,
+                int x_dtype, int w_dtype, float eps,
+                void* workspace, size_t workspace_bytes, void* counters, size_t counter_bytes,
+                void* stream);
+
+/* replaces _fused_rms_fwd, normalization/fused_rmsnorm_cached.py:389-501 (kernel :6-125):
+ * the two tensors are normalised in one launch as one virtual tensor; they share B and the dtype,
+ * and have independent T, C and weights. */
+int rgd_fused_rms_fwd(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2,
+                      const rgd_tensor3* x1, const rgd_tensor3* w1, const rgd_tensor3* y1,
+                      const rgd_tensor3* x2, const rgd_tensor3* w2, const rgd_tensor3* y2,
+                      int x_dtype, int w1_dtype, int w2_dtype, float eps, void* stream);
+
+/* replaces _fused_rms_bwd, normalization/fused_rmsnorm_cached.py:504-722 (kernels :128-319, :324-383) */
+int rgd_fused_rms_bwd(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2,
+                      const rgd_tensor3* dy1, const rgd_tensor3* x1, const rgd_tensor3* w1,
+                      const rgd_tensor3* dx1, const rgd_tensor3* dw1, int w1_shared,
+                      const rgd_tensor3* dy2, const rgd_tensor3* x2, const rgd_tensor3* w2,
+                      const rgd_tensor3* dx2, const rgd_tensor3* dw2, int w2_shared,
+                      int x_dtype, int w1_dtype, int w2_dtype, float eps,
+                      void* workspace, size_t workspace_bytes, void* counters, size_t counter_bytes,
+                      void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * L2 normalize  y = x / max(||x||, eps)              x (B,T,C)
+ * ------------------------------------------------------------------------------------------ */
+
+/* replaces _norm_fwd, normalization/l2normalize_cached.py:238-318 (kernel :5-124) */
+int rgd_l2_fwd(int64_t B, int64_t T, int64_t C, const rgd_tensor3* x, const rgd_tensor3* y,
+               int dtype, float eps, void* stream);
+
+/* replaces _norm_bwd, normalization/l2normalize_cached.py:321-399 (kernel :130-234):
+ *   dx = (dy - xhat*sum(xhat*dy)) * rlen, also for rows clamped by eps */
+int rgd_l2_bwd(int64_t B, int64_t T, int64_t C, const rgd_tensor3* dy, const rgd_tensor3* x,
+               const rgd_tensor3* dx, int dtype, float eps, void* stream);
+
+/* replaces _fused_norm_fwd, normalization/fused_l2normalize_cached.py:251-351 (kernel :6-115) */
+int rgd_fused_l2_fwd(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2,
+                     const rgd_tensor3* x1, const rgd_tensor3* y1,
+                     const rgd_tensor3* x2, const rgd_tensor3* y2,
+                     int dtype, float eps, void* stream);
+
+/* replaces _fused_norm_bwd, normalization/fused_l2normalize_cached.py:354-461 (kernel :121-247) */
+int rgd_fused_l2_bwd(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2,
+                     const rgd_tensor3* dy1, const rgd_tensor3* x1, const rgd_tensor3* dx1,
+                     const rgd_tensor3* dy2, const rgd_tensor3* x2, const rgd_tensor3* dx2,
+                     int dtype, float eps, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Per-head operators on query and key: q (B,H,Tq,D), k (B,H,Tk,D), one launch for both
+ * ------------------------------------------------------------------------------------------ */
+
+/* replaces _fused_ln_qk_fwd, normalization/head_layernorm_cached.py:204-309 (kernel :6-99):
+ * LayerNorm over D without affine, D <= 256 */
+int rgd_ln_qk_fwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D,
+                  const rgd_tensor4* q, const rgd_tensor4* k,
+                  const rgd_tensor4* qo, const rgd_tensor4* ko,
+                  int dtype, float eps, void* stream);
+
+/* replaces _fused_ln_qk_bwd, normalization/head_layernorm_cached.py:311-413 (kernel :101-202):
+ *   dx = (dy - xhat*mean(xhat*dy) - mean(dy)) * rstd; mean and rstd are recomputed from q, k */
+int rgd_ln_qk_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D,
+                  const rgd_tensor4* q, const rgd_tensor4* k,
+                  const rgd_tensor4* dqo, const rgd_tensor4* dko,
+                  const rgd_tensor4* dq, const rgd_tensor4* dk,
+                  int dtype, float eps, void* stream);
+
+/* replaces combined_rope_fn, rope/head_rope_cached.py:160-274 (kernel :56-158, helper :7-52):
+ *   out = x*cos + rot(x)*sin on channels < R of tokens < cutoff, copy elsewhere.
+ * pos_emb is (2, P, R): [0] = sin, [1] = cos, strides pe_stride_s / pe_stride_n, dtype pe_dtype.
+ * is_bwd flips the rotation sign (the reference's backward).  D <= 128, Tq < P and Tk < P.
+ * Arithmetic is fp32 with one rounding to the tensor dtype.  In-place (qo == q) is allowed. */
+int rgd_rope_qk(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D,
+                const rgd_tensor4* q, const rgd_tensor4* k,
+                const rgd_tensor4* qo, const rgd_tensor4* ko,
+                const void* pos_emb, int64_t P, int64_t R, int64_t pe_stride_s, int64_t pe_stride_n,
+                int pe_dtype, int64_t q_cutoff, int64_t k_cutoff, int is_bwd,
+                int dtype, void* stream);
+
+/* replaces _fused_rope_ln_qk_fwd, rope/fused_ln_rope_cached.py:382-516 (kernel :117-240) */
+int rgd_ln_rope_qk_fwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D,
+                       const rgd_tensor4* q, const rgd_tensor4* k,
+                       const rgd_tensor4* qo, const rgd_tensor4* ko,
+                       const void* pos_emb, int64_t P, int64_t R, int64_t pe_stride_s,
+                       int64_t pe_stride_n, int pe_dtype, int64_t q_cutoff, int64_t k_cutoff,
+                       int dtype, float eps, void* stream);
+
+/* replaces _fused_rope_ln_qk_bwd, rope/fused_ln_rope_cached.py:518-647 (kernel :243-378):
+ * inverse rotation of the upstream gradient, then the LayerNorm backward */
+int rgd_ln_rope_qk_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D,
+                       const rgd_tensor4* q, const rgd_tensor4* k,
+                       const rgd_tensor4* dqo, const rgd_tensor4* dko,
+                       const rgd_tensor4* dq, const rgd_tensor4* dk,
+                       const void* pos_emb, int64_t P, int64_t R, int64_t pe_stride_s,
+                       int64_t pe_stride_n, int pe_dtype, int64_t q_cutoff, int64_t k_cutoff,
+                       int dtype, float eps, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Attention with additive bias: q (B,Tq,H,D), k,v (B,Tk,H,D) given as (b,h,n) strides, D <= 128,
+ * fp16 or bf16.  bias (B,H,Tq,Tk) by strides (stride_n = row stride; 0 rows for RGD_BIAS_VECTOR),
+ * dtype = the tensor dtype or fp32, zero strides broadcast.
+ * ------------------------------------------------------------------------------------------ */
+
+/* rows of the LSE / delta buffers: Tq rounded up to a multiple of 64, as the reference allocates
+ * them (flash_attn/flash_attn_triton_cached.py:790-792) */
+int64_t rgd_attn_seqlen_q_rounded(int64_t Tq);
+
+/* replaces _flash_attn_forward, flash_attn/flash_attn_triton_cached.py:758-882 (kernel :21-246).
+ * lse is fp32 (B, H, Tq_rounded); rows >= Tq are written as 0.  A query row whose logits are all
+ * -inf gives o = 0 and lse = -inf. */
+int rgd_attn_fwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D,
+                 const rgd_tensor4* q, const rgd_tensor4* k, const rgd_tensor4* v,
+                 const rgd_tensor4* bias, int bias_kind, int bias_dtype,
+                 const rgd_tensor4* o, float* lse,
+                 int dtype, int causal, float softmax_scale, void* stream);
+
+/* bytes of scratch rgd_attn_bwd needs (delta, fp32 (B,H,Tq_rounded)); any contents on entry */
+size_t rgd_attn_bwd_workspace(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D);
+
+/* replaces _flash_attn_backward, flash_attn/flash_attn_triton_cached.py:885-1075
+ * (kernels :249-292 and :327-755): delta = rowsum(o*do), P recomputed from lse, dv = P^T do,
+ * dS = P*(do v^T - delta)*scale, dk = dS^T q, dq = dS k.  No bias gradient.  dq, dk, dv are written
+ * in the tensor dtype from fp32 accumulators, each exactly once, in a fixed order. */
+int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D,
+                 const rgd_tensor4* dout, const rgd_tensor4* q, const rgd_tensor4* k,
+                 const rgd_tensor4* v, const rgd_tensor4* o, const float* lse,
+                 const rgd_tensor4* bias, int bias_kind, int bias_dtype,
+                 const rgd_tensor4* dq, const rgd_tensor4* dk, const rgd_tensor4* dv,
+                 int dtype, int causal, float softmax_scale,
+                 void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RGD_HIP_H */

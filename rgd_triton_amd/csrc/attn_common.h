@@ -1,0 +1,124 @@
+// Pieces shared by the attention kernels: the 32x32x16 MFMA wrappers, the row permutation that makes a
+// lane's 16 accumulator values contiguous, tile loaders and bias access.
+//
+// MFMA v_mfma_f32_32x32x16_{bf16,f16} on a 64-lane wavefront, D = A(32x16) * B(16x32) + C:
+//   A operand: lane l holds A[l%32][8*(l/32) .. +7]        (8 contiguous K values of one row)
+//   B operand: lane l holds B[8*(l/32) .. +7][l%32]        (8 contiguous K values of one column)
+//   C / D:     lane l holds column l%32, rows 8*(v/4) + 4*(l/32) + v%4 for v = 0..15
+// Which matrix row an MFMA row stands for is the kernel's choice (it only decides which address a
+// lane reads its A operand from).  All kernels here read MFMA row r = 8a + 4g + c from matrix row
+// perm(r) = 16g + 4a + c, so that lane (l%32, g = l/32) ends up holding the 16 CONTIGUOUS matrix rows
+// 16g .. 16g+15 of its column, in register order v = 0..15.  That makes bias loads, probability
+// operands and output stores 16-element contiguous runs per lane.
+#pragma once
+
+#include "common.h"
+
+template <typename T> struct Mfma;
+template <> struct Mfma<bf16_t> {
+    typedef bf16x8 V8;
+    static __device__ __forceinline__ f32x16 run(V8 a, V8 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+};
+template <> struct Mfma<f16_t> {
+    typedef f16x8 V8;
+    static __device__ __forceinline__ f32x16 run(V8 a, V8 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+};
+
+// matrix row read by MFMA row r (r = lane % 32 for an A operand)
+__device__ __forceinline__ int mfma_row_perm(int r) { return ((r >> 2) & 1) * 16 + (r >> 3) * 4 + (r & 3); }
+
+union Pack16 {  // 8 16-bit elements <-> one 16-byte vector
+    u32x4 v;
+    uint32_t w[4];
+    uint16_t h[8];
+};
+
+// 8 elements of a row starting at column `col`; columns >= ncols and rows flagged invalid read as 0.
+// `vec` = 16-byte access is legal for this tensor.
+template <typename T>
+__device__ __forceinline__ u32x4 load8(const T* __restrict__ row, int col, int ncols, bool valid, bool vec) {
+    Pack16 p;
+    p.v = u32x4{0u, 0u, 0u, 0u};
+    if (valid) {
+        if (vec) {
+            if (col < ncols) p.v = *reinterpret_cast<const u32x4*>(row + col);
+        } else {
+            const uint16_t* r16 = reinterpret_cast<const uint16_t*>(row);
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (col + e < ncols) p.h[e] = r16[col + e];
+        }
+    }
+    return p.v;
+}
+
+template <typename T> __device__ __forceinline__ typename Mfma<T>::V8 as_v8(u32x4 raw) {
+    return __builtin_bit_cast(typename Mfma<T>::V8, raw);
+}
+
+// two fp32 -> one dword of two T (round to nearest even)
+template <typename T> __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    typedef T T2 __attribute__((ext_vector_type(2)));
+    T2 t;
+    t[0] = static_cast<T>(lo);
+    t[1] = static_cast<T>(hi);
+    return __builtin_bit_cast(uint32_t, t);
+}
+
+// 16 contiguous bias values for one lane -> fp32, scaled by log2(e).  dtype is the bias element type.
+// `vec` = the run is 16-byte aligned and fully in range; otherwise elements >= limit read as 0.
+__device__ __forceinline__ void load_bias16(const void* base, int64_t off, int dtype, int first, int limit, bool vec,
+                                            float scale, float (&out)[16]) {
+    if (dtype == RGD_F32) {
+        const float* p = static_cast<const float*>(base) + off;
+        if (vec) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                f32x4 t = *reinterpret_cast<const f32x4*>(p + first + 4 * i);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) out[4 * i + e] = t[e] * scale;
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) out[e] = (first + e < limit) ? p[first + e] * scale : 0.f;
+        }
+    } else {
+        const uint16_t* p = static_cast<const uint16_t*>(base) + off;
+        Pack16 a, b;
+        if (vec) {
+            a.v = *reinterpret_cast<const u32x4*>(p + first);
+            b.v = *reinterpret_cast<const u32x4*>(p + first + 8);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                a.h[e] = (first + e < limit) ? p[first + e] : (uint16_t)0;
+                b.h[e] = (first + 8 + e < limit) ? p[first + 8 + e] : (uint16_t)0;
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            float x, y;
+            if (dtype == RGD_BF16) {
+                x = __builtin_bit_cast(float, (uint32_t)a.h[e] << 16);
+                y = __builtin_bit_cast(float, (uint32_t)b.h[e] << 16);
+            } else {
+                x = static_cast<float>(__builtin_bit_cast(f16_t, a.h[e]));
+                y = static_cast<float>(__builtin_bit_cast(f16_t, b.h[e]));
+            }
+            out[e] = x * scale;
+            out[8 + e] = y * scale;
+        }
+    }
+}
+
+struct AttnTensor {
+    const void* ptr;
+    int64_t sb, sh, sn;
+};
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;

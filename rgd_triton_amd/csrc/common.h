@@ -1,0 +1,195 @@
+// Shared host/device helpers for the gfx950 kernels: error reporting, dtype traits,
+// 16-byte vector access, wavefront (64-lane) group reductions on DPP / ds_swizzle, fast division.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/rgd_hip.h"
+
+// ------------------------------------------------------------------------------------------
+// host: errors
+// ------------------------------------------------------------------------------------------
+void rgd_set_error(const char* fmt, ...);  // defined in api.hip
+
+#define RGD_REQUIRE(cond, code, ...)        \
+    do {                                    \
+        if (!(cond)) {                      \
+            rgd_set_error(__VA_ARGS__);     \
+            return (code);                  \
+        }                                   \
+    } while (0)
+
+#define RGD_CHECK_LAUNCH(name)                                                        \
+    do {                                                                              \
+        hipError_t e_ = hipGetLastError();                                            \
+        if (e_ != hipSuccess) {                                                       \
+            rgd_set_error("%s: kernel launch failed: %s", name, hipGetErrorString(e_)); \
+            return RGD_ERR_LAUNCH;                                                    \
+        }                                                                             \
+    } while (0)
+
+static inline bool rgd_dtype_ok(int d) { return d == RGD_F32 || d == RGD_F16 || d == RGD_BF16; }
+static inline int rgd_dtype_size(int d) { return d == RGD_F32 ? 4 : 2; }
+static inline bool rgd_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ------------------------------------------------------------------------------------------
+// element types
+// ------------------------------------------------------------------------------------------
+typedef _Float16 f16_t;
+typedef __bf16 bf16_t;
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef bf16_t bf16x8 __attribute__((ext_vector_type(8)));
+typedef f16_t f16x8 __attribute__((ext_vector_type(8)));
+typedef bf16_t bf16x4 __attribute__((ext_vector_type(4)));
+typedef f16_t f16x4 __attribute__((ext_vector_type(4)));
+
+template <typename T> struct DType;
+template <> struct DType<float> { static constexpr int code = RGD_F32; };
+template <> struct DType<f16_t> { static constexpr int code = RGD_F16; };
+template <> struct DType<bf16_t> { static constexpr int code = RGD_BF16; };
+
+template <typename T> __device__ __forceinline__ float to_f32(T v) { return static_cast<float>(v); }
+template <typename T> __device__ __forceinline__ T from_f32(float v) { return static_cast<T>(v); }
+
+// ------------------------------------------------------------------------------------------
+// chunk access: N contiguous elements of type T <-> N floats.
+// VECTOR = true uses 16-byte accesses (address and N*sizeof(T) must be multiples of 16).
+// ------------------------------------------------------------------------------------------
+template <typename T, int N, bool VECTOR>
+__device__ __forceinline__ void load_chunk(const T* __restrict__ p, int first, int limit, float (&out)[N]) {
+    // loads elements [first, first+N) of the row at p; elements at or beyond `limit` read as 0
+    // a chunk that is not a whole number of 16-byte vectors (fp32 rows with 16-bit weights) is read
+    // element by element
+    if constexpr (VECTOR && (N * sizeof(T)) % 16 == 0) {
+        constexpr int BYTES = N * sizeof(T);
+        constexpr int NV = BYTES / 16;
+        constexpr int EPV = 16 / sizeof(T);
+        if (first < limit) {  // limit is a multiple of N on this path
+            const u32x4* vp = reinterpret_cast<const u32x4*>(p + first);
+#pragma unroll
+            for (int v = 0; v < NV; ++v) {
+                u32x4 raw = vp[v];
+                T tmp[EPV];
+                __builtin_memcpy(tmp, &raw, 16);
+#pragma unroll
+                for (int e = 0; e < EPV; ++e) out[v * EPV + e] = to_f32<T>(tmp[e]);
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < N; ++e) out[e] = 0.f;
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < N; ++e) out[e] = (first + e < limit) ? to_f32<T>(p[first + e]) : 0.f;
+    }
+}
+
+template <typename T, int N, bool VECTOR>
+__device__ __forceinline__ void store_chunk(T* __restrict__ p, int first, int limit, const float (&in)[N]) {
+    if constexpr (VECTOR && (N * sizeof(T)) % 16 == 0) {
+        constexpr int BYTES = N * sizeof(T);
+        constexpr int NV = BYTES / 16;
+        constexpr int EPV = 16 / sizeof(T);
+        if (first < limit) {
+            u32x4* vp = reinterpret_cast<u32x4*>(p + first);
+#pragma unroll
+            for (int v = 0; v < NV; ++v) {
+                T tmp[EPV];
+#pragma unroll
+                for (int e = 0; e < EPV; ++e) tmp[e] = from_f32<T>(in[v * EPV + e]);
+                u32x4 raw;
+                __builtin_memcpy(&raw, tmp, 16);
+                vp[v] = raw;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < N; ++e)
+            if (first + e < limit) p[first + e] = from_f32<T>(in[e]);
+    }
+}
+
+// chunk load whose element type is only known at run time (weights, rotary tables)
+template <int N, bool VECTOR>
+__device__ __forceinline__ void load_chunk_dyn(const void* p, int dtype, int first, int limit, float (&out)[N]) {
+    if (dtype == RGD_BF16)
+        load_chunk<bf16_t, N, VECTOR>(static_cast<const bf16_t*>(p), first, limit, out);
+    else if (dtype == RGD_F16)
+        load_chunk<f16_t, N, VECTOR>(static_cast<const f16_t*>(p), first, limit, out);
+    else
+        load_chunk<float, N, VECTOR>(static_cast<const float*>(p), first, limit, out);
+}
+
+__device__ __forceinline__ void store_dyn(void* p, int dtype, int64_t idx, float v) {
+    if (dtype == RGD_BF16)
+        static_cast<bf16_t*>(p)[idx] = from_f32<bf16_t>(v);
+    else if (dtype == RGD_F16)
+        static_cast<f16_t*>(p)[idx] = from_f32<f16_t>(v);
+    else
+        static_cast<float*>(p)[idx] = v;
+}
+
+// ------------------------------------------------------------------------------------------
+// wavefront group reductions.  A "group" is G consecutive lanes (G a power of two <= 64);
+// every lane of the group ends up with the group's result.
+// ------------------------------------------------------------------------------------------
+template <int CTRL> __device__ __forceinline__ float dpp_move(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float lane_xor16(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));  // SWAP,16
+}
+__device__ __forceinline__ float lane_xor32(float v) {
+    int lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, __builtin_bit_cast(int, v)));
+}
+
+struct OpSum { static __device__ __forceinline__ float apply(float a, float b) { return a + b; } };
+struct OpMax { static __device__ __forceinline__ float apply(float a, float b) { return fmaxf(a, b); } };
+
+template <int G, typename Op = OpSum> __device__ __forceinline__ float group_reduce(float v) {
+    // quad_perm [1,0,3,2] / [2,3,0,1], then row_half_mirror and row_mirror: after the quad steps all
+    // four lanes of a quad agree, so the mirrors are equivalent to xor 4 and xor 8
+    if constexpr (G >= 2) v = Op::apply(v, dpp_move<0xB1>(v));
+    if constexpr (G >= 4) v = Op::apply(v, dpp_move<0x4E>(v));
+    if constexpr (G >= 8) v = Op::apply(v, dpp_move<0x141>(v));
+    if constexpr (G >= 16) v = Op::apply(v, dpp_move<0x140>(v));
+    if constexpr (G >= 32) v = Op::apply(v, lane_xor16(v));
+    if constexpr (G >= 64) v = Op::apply(v, lane_xor32(v));
+    return v;
+}
+
+// sum over the lanes of a wave that share (lane % G): used once per block for the dw partials
+template <int G> __device__ __forceinline__ float cross_group_sum(float v) {
+#pragma unroll
+    for (int off = G; off < 64; off <<= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+// ------------------------------------------------------------------------------------------
+// division of a 31-bit value by a run-time constant: q = (mulhi(n, m) + n) >> s
+// ------------------------------------------------------------------------------------------
+struct FastDiv {
+    uint32_t d, m, s;
+};
+static inline FastDiv make_fastdiv(uint32_t d) {
+    FastDiv f;
+    f.d = d ? d : 1;
+    uint32_t s = 0;
+    while ((1ull << s) < f.d) ++s;
+    f.s = s;
+    f.m = static_cast<uint32_t>(((1ull << 32) * ((1ull << s) - f.d)) / f.d + 1);
+    return f;
+}
+__device__ __forceinline__ uint32_t fast_div(uint32_t n, const FastDiv& f) {
+    return (__umulhi(n, f.m) + n) >> f.s;
+}
+
+__device__ __forceinline__ int lane_id() { return __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); }

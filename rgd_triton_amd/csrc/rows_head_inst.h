@@ -1,0 +1,42 @@
+// Instantiates head_rows_kernel for one element type and dispatches a run-time configuration to it.
+#pragma once
+
+#include "rows_head.h"
+
+template <typename T, int MODE, int G, int NV, bool VECTOR>
+static int head_launch_one(const HeadParams& p, dim3 grid, hipStream_t s) {
+    constexpr int VEC = VECTOR ? 16 / (int)sizeof(T) : 2;
+    constexpr int U = head_unroll(MODE, NV);
+    hipLaunchKernelGGL((head_rows_kernel<T, MODE, G, NV, VEC, VECTOR, U>), grid, dim3(256), 0, s, p);
+    return 0;
+}
+
+template <typename T, int MODE, bool VECTOR>
+static int head_dispatch_shape(const HeadConfig& c, const HeadParams& p, dim3 grid, hipStream_t s) {
+#define HEAD_CASE(g, nv) \
+    if (c.G == g && c.NV == nv) return head_launch_one<T, MODE, g, nv, VECTOR>(p, grid, s);
+    HEAD_CASE(4, 1)
+    HEAD_CASE(8, 1)
+    HEAD_CASE(16, 1)
+    HEAD_CASE(32, 1)
+    HEAD_CASE(64, 1)
+    HEAD_CASE(64, 2)
+#undef HEAD_CASE
+    rgd_set_error("head rows: no kernel for G=%d NV=%d", c.G, c.NV);
+    return RGD_ERR_UNSUPPORTED;
+}
+
+template <typename T> int head_dispatch(const HeadConfig& c, const HeadParams& p, dim3 grid, hipStream_t s) {
+#define HEAD_MODE(m)                                                                \
+    if (c.mode == m)                                                                \
+        return c.vector ? head_dispatch_shape<T, m, true>(c, p, grid, s)            \
+                        : head_dispatch_shape<T, m, false>(c, p, grid, s);
+    HEAD_MODE(HEAD_LN_FWD)
+    HEAD_MODE(HEAD_LN_BWD)
+    HEAD_MODE(HEAD_ROPE)
+    HEAD_MODE(HEAD_LNROPE_FWD)
+    HEAD_MODE(HEAD_LNROPE_BWD)
+#undef HEAD_MODE
+    rgd_set_error("head rows: bad mode %d", c.mode);
+    return RGD_ERR_INVALID;
+}

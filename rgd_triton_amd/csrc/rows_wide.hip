@@ -1,0 +1,294 @@
+// Host side of the (B,T,C) row kernels: argument validation, configuration choice, workspace layout
+// and the extern "C" entry points for RMSNorm / RMSNorm2 / L2 / L2x2.
+#include "rows_wide.h"
+
+#include <algorithm>
+#include <string.h>
+
+int rgd_num_cus();  // api.hip
+
+namespace {
+
+constexpr int DW_BLOCKS_PER_CU = 1;  // leaves of the dw tree per compute unit (RMSNorm backward)
+constexpr int BLOCKS_PER_CU = 8;     // target grid size of the other kernels
+
+int pow2ceil(int v) {
+    int p = 1;
+    while (p < v) p <<= 1;
+    return p;
+}
+
+struct TreeShape {
+    int rows = 0, ctrs = 0;
+    int row_off[WIDE_MAX_LEVELS] = {0}, ctr_off[WIDE_MAX_LEVELS] = {0};
+};
+
+TreeShape tree_shape(int nleaf) {
+    TreeShape t;
+    int n = nleaf, lvl = 0;
+    while (n > 1 && lvl < WIDE_MAX_LEVELS) {
+        t.row_off[lvl] = t.rows;
+        t.ctr_off[lvl] = t.ctrs;
+        t.rows += n;
+        n = (n + WIDE_FANIN - 1) / WIDE_FANIN;
+        t.ctrs += n;
+        ++lvl;
+    }
+    if (lvl < WIDE_MAX_LEVELS) t.row_off[lvl] = t.rows;
+    return t;
+}
+
+// upper bound of partial rows / counters one half can need, whatever tile shape is chosen later
+void half_bound(int64_t B, int64_t T, int64_t target, size_t* rows, size_t* ctrs) {
+    if (T <= 0) {
+        *rows = *ctrs = 0;
+        return;
+    }
+    const size_t leaves = (size_t)target + (size_t)B;
+    *rows = leaves + leaves / 8 + 8 * (size_t)B + 8;
+    *ctrs = leaves / 8 + 8 * (size_t)B + 8;
+}
+
+bool t3_vec_ok(const rgd_tensor3* t, int es) {
+    return t && rgd_aligned16(t->ptr) && (t->stride_b * es) % 16 == 0 && (t->stride_n * es) % 16 == 0;
+}
+
+}  // namespace
+
+int wide_workspace(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2, size_t* ws, size_t* ctr) {
+    const int64_t target = (int64_t)rgd_num_cus() * DW_BLOCKS_PER_CU;
+    size_t r1, c1, r2, c2;
+    half_bound(B, T1, target, &r1, &c1);
+    half_bound(B, T2, target, &r2, &c2);
+    *ws = (r1 * (size_t)std::max<int64_t>(C1, 0) + r2 * (size_t)std::max<int64_t>(C2, 0)) * sizeof(float);
+    *ctr = (c1 + c2) * sizeof(int);
+    return RGD_OK;
+}
+
+int wide_launch(const char* name, int op, bool bwd, int64_t B, const WideHalfArgs& a1, const WideHalfArgs& a2,
+                int dtype, float eps, void* workspace, size_t workspace_bytes, void* counters,
+                size_t counter_bytes, void* stream) {
+    RGD_REQUIRE(rgd_dtype_ok(dtype), RGD_ERR_INVALID, "%s: Only support fp16, bf16, and fp32", name);
+    RGD_REQUIRE(B >= 0 && B <= 65535, RGD_ERR_INVALID, "%s: batch %lld out of range", name, (long long)B);
+    const WideHalfArgs* as[2] = {&a1, &a2};
+    const int es = rgd_dtype_size(dtype);
+    const bool has_w = op == WIDE_RMS;
+    bool vector = true;
+    int64_t maxC = 0, total_rows = 0;
+    for (const WideHalfArgs* a : as) {
+        RGD_REQUIRE(a->T >= 0 && a->T < (1ll << 31) && a->C >= 0 && a->C < (1ll << 31), RGD_ERR_INVALID,
+                    "%s: shape out of range", name);
+        if (a->T == 0 || a->C == 0) continue;
+        RGD_REQUIRE(a->x && a->x->ptr && a->y && a->y->ptr, RGD_ERR_INVALID, "%s: null tensor", name);
+        RGD_REQUIRE(!bwd || (a->dy && a->dy->ptr), RGD_ERR_INVALID, "%s: null gradient", name);
+        RGD_REQUIRE(!has_w || (a->w && a->w->ptr && rgd_dtype_ok(a->w_dtype)), RGD_ERR_INVALID, "%s: bad weight", name);
+        RGD_REQUIRE(!(has_w && bwd) || (a->dw && a->dw->ptr), RGD_ERR_INVALID, "%s: null dw", name);
+        vector = vector && (a->C * es) % 16 == 0 && t3_vec_ok(a->x, es) && t3_vec_ok(a->y, es) &&
+                 (!bwd || t3_vec_ok(a->dy, es));
+        maxC = std::max(maxC, a->C);
+        total_rows += B * a->T;
+    }
+    if (total_rows == 0 || B == 0) return RGD_OK;
+
+    WideConfig cfg;
+    cfg.op = op;
+    cfg.bwd = bwd;
+    cfg.vector = vector;
+    const int vec = vector ? 16 / es : 2;
+    const int64_t chunks = (maxC + vec - 1) / vec;
+    if (chunks <= 64) {
+        cfg.G = std::max(4, pow2ceil((int)chunks));
+        cfg.NV = 1;
+    } else {
+        static const int allowed[] = {2, 3, 4, 6, 8, 12, 16};
+        const int64_t need = (chunks + 63) / 64;
+        cfg.G = 64;
+        cfg.NV = 0;
+        for (int nv : allowed)
+            if (nv >= need) {
+                cfg.NV = nv;
+                break;
+            }
+        RGD_REQUIRE(cfg.NV != 0, RGD_ERR_UNSUPPORTED,
+                    "%s: rows of %lld elements exceed the register-resident limit (%d)", name, (long long)maxC,
+                    64 * 16 * vec);
+    }
+    const int NW = wide_waves(op, bwd);
+    const int U = wide_unroll(bwd, cfg.NV);
+    const int row_quantum = NW * (64 / cfg.G) * U;
+    const bool tree = has_w && bwd;
+    const int64_t target = (int64_t)rgd_num_cus() * (tree ? DW_BLOCKS_PER_CU : BLOCKS_PER_CU);
+    int64_t rpc = (total_rows + target - 1) / target;
+    rpc = std::max<int64_t>(row_quantum, (rpc + row_quantum - 1) / row_quantum * row_quantum);
+    RGD_REQUIRE(rpc < (1ll << 30), RGD_ERR_UNSUPPORTED, "%s: too many rows", name);
+
+    WideParams p;
+    memset(&p, 0, sizeof(p));
+    p.rows_per_chunk = (int)rpc;
+    p.eps = eps;
+    size_t ws_used = 0, ctr_used = 0;
+    int64_t grid_x = 0;
+    for (int i = 0; i < 2; ++i) {
+        const WideHalfArgs* a = as[i];
+        WideHalf& h = p.h[i];
+        if (a->T == 0 || a->C == 0) {
+            h.nchunks = 0;
+            continue;
+        }
+        h.x = a->x->ptr;
+        h.sx_b = a->x->stride_b;
+        h.sx_n = a->x->stride_n;
+        h.y = a->y->ptr;
+        h.sy_b = a->y->stride_b;
+        h.sy_n = a->y->stride_n;
+        if (bwd) {
+            h.dy = a->dy->ptr;
+            h.sd_b = a->dy->stride_b;
+            h.sd_n = a->dy->stride_n;
+        }
+        h.T = (int)a->T;
+        h.C = (int)a->C;
+        h.inv_c = 1.0f / (float)a->C;
+        h.nchunks = (int)((a->T + rpc - 1) / rpc);
+        grid_x += h.nchunks;
+        if (has_w) {
+            const int ws_ = rgd_dtype_size(a->w_dtype);
+            h.w = a->w->ptr;
+            h.sw_b = a->w->stride_b;
+            h.w_dtype = a->w_dtype;
+            h.w_vec = rgd_aligned16(a->w->ptr) && (a->w->stride_b * ws_) % 16 == 0 && (a->C * ws_) % 16 == 0 &&
+                      (vec * ws_) % 16 == 0;
+        }
+        if (tree) {
+            h.dw = a->dw->ptr;
+            h.sdw_b = a->dw->stride_b;
+            h.w_shared = a->w_shared ? 1 : 0;
+            h.nleaf = h.w_shared ? (int)B * h.nchunks : h.nchunks;
+            const int ntrees = h.w_shared ? 1 : (int)B;
+            const TreeShape ts = tree_shape(h.nleaf);
+            h.tree_rows = ts.rows;
+            h.tree_ctrs = ts.ctrs;
+            for (int l = 0; l < WIDE_MAX_LEVELS; ++l) {
+                h.lvl_row_off[l] = ts.row_off[l];
+                h.lvl_ctr_off[l] = ts.ctr_off[l];
+            }
+            h.part = reinterpret_cast<float*>(static_cast<char*>(workspace) + ws_used);
+            h.ctr = reinterpret_cast<int*>(static_cast<char*>(counters) + ctr_used);
+            ws_used += (size_t)ntrees * ts.rows * a->C * sizeof(float);
+            ctr_used += (size_t)ntrees * ts.ctrs * sizeof(int);
+        }
+    }
+    if (tree) {
+        RGD_REQUIRE(ws_used <= workspace_bytes && ctr_used <= counter_bytes, RGD_ERR_WORKSPACE,
+                    "%s: workspace too small (need %zu + %zu bytes, have %zu + %zu)", name, ws_used, ctr_used,
+                    workspace_bytes, counter_bytes);
+        RGD_REQUIRE((ws_used == 0 || workspace) && (ctr_used == 0 || counters), RGD_ERR_INVALID,
+                    "%s: null workspace", name);
+    }
+    RGD_REQUIRE(grid_x < (1ll << 31), RGD_ERR_UNSUPPORTED, "%s: grid too large", name);
+
+    const dim3 grid((unsigned)grid_x, (unsigned)B, 1);
+    const size_t lds = tree ? (size_t)maxC * sizeof(float) : 0;
+    RGD_REQUIRE(lds <= 64 * 1024, RGD_ERR_UNSUPPORTED, "%s: row too wide for the dw staging buffer", name);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    int rc;
+    if (dtype == RGD_F32)
+        rc = wide_dispatch<float>(cfg, p, grid, lds, s);
+    else if (dtype == RGD_F16)
+        rc = wide_dispatch<f16_t>(cfg, p, grid, lds, s);
+    else
+        rc = wide_dispatch<bf16_t>(cfg, p, grid, lds, s);
+    if (rc != RGD_OK) return rc;
+    RGD_CHECK_LAUNCH(name);
+    return RGD_OK;
+}
+
+// ------------------------------------------------------------------------------------------
+// C ABI
+// ------------------------------------------------------------------------------------------
+namespace {
+WideHalfArgs half(int64_t T, int64_t C, const rgd_tensor3* x, const rgd_tensor3* dy, const rgd_tensor3* y,
+                  const rgd_tensor3* w = nullptr, const rgd_tensor3* dw = nullptr, int w_dtype = RGD_F32,
+                  int w_shared = 0) {
+    WideHalfArgs a;
+    a.T = T;
+    a.C = C;
+    a.x = x;
+    a.dy = dy;
+    a.y = y;
+    a.w = w;
+    a.dw = dw;
+    a.w_dtype = w_dtype;
+    a.w_shared = w_shared;
+    return a;
+}
+const WideHalfArgs kNoHalf;
+}  // namespace
+
+extern "C" {
+
+int rgd_rms_fwd(int64_t B, int64_t T, int64_t C, const rgd_tensor3* x, const rgd_tensor3* w, const rgd_tensor3* y,
+                int x_dtype, int w_dtype, float eps, void* stream) {
+    return wide_launch("rgd_rms_fwd", WIDE_RMS, false, B, half(T, C, x, nullptr, y, w, nullptr, w_dtype), kNoHalf,
+                       x_dtype, eps, nullptr, 0, nullptr, 0, stream);
+}
+
+int rgd_rms_bwd_workspace(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2, size_t* workspace_bytes,
+                          size_t* counter_bytes) {
+    RGD_REQUIRE(workspace_bytes && counter_bytes, RGD_ERR_INVALID, "rgd_rms_bwd_workspace: null output");
+    return wide_workspace(B, T1, C1, T2, C2, workspace_bytes, counter_bytes);
+}
+
+int rgd_rms_bwd(int64_t B, int64_t T, int64_t C, const rgd_tensor3* dy, const rgd_tensor3* x, const rgd_tensor3* w,
+                const rgd_tensor3* dx, const rgd_tensor3* dw, int w_shared, int x_dtype, int w_dtype, float eps,
+                void* workspace, size_t workspace_bytes, void* counters, size_t counter_bytes, void* stream) {
+    return wide_launch("rgd_rms_bwd", WIDE_RMS, true, B, half(T, C, x, dy, dx, w, dw, w_dtype, w_shared), kNoHalf,
+                       x_dtype, eps, workspace, workspace_bytes, counters, counter_bytes, stream);
+}
+
+int rgd_fused_rms_fwd(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2, const rgd_tensor3* x1,
+                      const rgd_tensor3* w1, const rgd_tensor3* y1, const rgd_tensor3* x2, const rgd_tensor3* w2,
+                      const rgd_tensor3* y2, int x_dtype, int w1_dtype, int w2_dtype, float eps, void* stream) {
+    return wide_launch("rgd_fused_rms_fwd", WIDE_RMS, false, B, half(T1, C1, x1, nullptr, y1, w1, nullptr, w1_dtype),
+                       half(T2, C2, x2, nullptr, y2, w2, nullptr, w2_dtype), x_dtype, eps, nullptr, 0, nullptr, 0,
+                       stream);
+}
+
+int rgd_fused_rms_bwd(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2, const rgd_tensor3* dy1,
+                      const rgd_tensor3* x1, const rgd_tensor3* w1, const rgd_tensor3* dx1, const rgd_tensor3* dw1,
+                      int w1_shared, const rgd_tensor3* dy2, const rgd_tensor3* x2, const rgd_tensor3* w2,
+                      const rgd_tensor3* dx2, const rgd_tensor3* dw2, int w2_shared, int x_dtype, int w1_dtype,
+                      int w2_dtype, float eps, void* workspace, size_t workspace_bytes, void* counters,
+                      size_t counter_bytes, void* stream) {
+    return wide_launch("rgd_fused_rms_bwd", WIDE_RMS, true, B, half(T1, C1, x1, dy1, dx1, w1, dw1, w1_dtype, w1_shared),
+                       half(T2, C2, x2, dy2, dx2, w2, dw2, w2_dtype, w2_shared), x_dtype, eps, workspace,
+                       workspace_bytes, counters, counter_bytes, stream);
+}
+
+int rgd_l2_fwd(int64_t B, int64_t T, int64_t C, const rgd_tensor3* x, const rgd_tensor3* y, int dtype, float eps,
+               void* stream) {
+    return wide_launch("rgd_l2_fwd", WIDE_L2, false, B, half(T, C, x, nullptr, y), kNoHalf, dtype, eps, nullptr, 0,
+                       nullptr, 0, stream);
+}
+
+int rgd_l2_bwd(int64_t B, int64_t T, int64_t C, const rgd_tensor3* dy, const rgd_tensor3* x, const rgd_tensor3* dx,
+               int dtype, float eps, void* stream) {
+    return wide_launch("rgd_l2_bwd", WIDE_L2, true, B, half(T, C, x, dy, dx), kNoHalf, dtype, eps, nullptr, 0, nullptr,
+                       0, stream);
+}
+
+int rgd_fused_l2_fwd(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2, const rgd_tensor3* x1,
+                     const rgd_tensor3* y1, const rgd_tensor3* x2, const rgd_tensor3* y2, int dtype, float eps,
+                     void* stream) {
+    return wide_launch("rgd_fused_l2_fwd", WIDE_L2, false, B, half(T1, C1, x1, nullptr, y1),
+                       half(T2, C2, x2, nullptr, y2), dtype, eps, nullptr, 0, nullptr, 0, stream);
+}
+
+int rgd_fused_l2_bwd(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2, const rgd_tensor3* dy1,
+                     const rgd_tensor3* x1, const rgd_tensor3* dx1, const rgd_tensor3* dy2, const rgd_tensor3* x2,
+                     const rgd_tensor3* dx2, int dtype, float eps, void* stream) {
+    return wide_launch("rgd_fused_l2_bwd", WIDE_L2, true, B, half(T1, C1, x1, dy1, dx1), half(T2, C2, x2, dy2, dx2),
+                       dtype, eps, nullptr, 0, nullptr, 0, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,46 @@
+"""Shared pieces of the parity tests: seeded CPU input generation (the oracle and the GPU kernel see
+the same bits) and the reference's comparison rules."""
+import os
+import sys
+
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "oracle"))
+
+import rgd_oracle as oracle  # noqa: E402
+
+DTYPES = [torch.float32, torch.float16, torch.bfloat16]
+DEV = "cuda"
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def randn(g, *shape, dtype=torch.float32, scale=1.0, shift=0.0):
+    """N(shift, scale) drawn on the CPU in fp32, then rounded to dtype."""
+    return (torch.randn(*shape, generator=g, dtype=torch.float32) * scale + shift).to(dtype)
+
+
+def to_gpu(*ts, requires_grad=False):
+    out = [t.to(DEV).detach().requires_grad_(requires_grad) for t in ts]
+    return out if len(out) > 1 else out[0]
+
+
+def assert_close(actual, expected, dtype, op="default", name="", atol_scale=1.0):
+    rtol, atol = oracle.get_tolerance(dtype, op)
+    torch.testing.assert_close(actual.detach().cpu(), expected.detach().cpu(), rtol=rtol, atol=atol * atol_scale,
+                               msg=lambda m: f"{name}: {m}")
+
+
+def assert_close_allow_inf(actual, expected, dtype, name=""):
+    """safe_assert_close_allow_inf of the reference's L2 tests (tests/test_l2normalize.py:54-111):
+    NaN is forbidden, +-inf must sit at the same places, finite values compare within tolerance."""
+    a, e = actual.detach().cpu().float(), expected.detach().cpu().float()
+    assert not torch.isnan(a).any(), f"{name}: NaN in result"
+    assert torch.equal(torch.isinf(a), torch.isinf(e)), f"{name}: inf pattern differs"
+    fin = ~torch.isinf(e)
+    rtol, atol = oracle.get_tolerance(dtype)
+    torch.testing.assert_close(a[fin], e[fin], rtol=rtol, atol=atol, msg=lambda m: f"{name}: {m}")

@@ -1,0 +1,232 @@
+"""GPU parity of FusedHeadLayerNorm, RoPE and FusedLNRoPE.  Counterparts of the reference's
+tests/test_head_layernorm.py, tests/test_head_rope.py and tests/test_fused_ln_rope.py."""
+import pytest
+import torch
+
+from helpers import DTYPES, assert_close, gen, oracle, randn, to_gpu
+
+pytestmark = pytest.mark.gpu
+
+SEQ_PAIRS = [(31, 11), (23, 138), (113, 203), (128, 217), (108, 256), (256, 512), (1023, 1024), (1, 239), (239, 1)]
+D_R = [(32, 32), (64, 32), (64, 64), (128, 32), (128, 64), (128, 96), (128, 128)]
+
+
+def _qk(g, B, H, Tq, Tk, D, dtype, heads_second, shift=0.0, scale=1.0):
+    if heads_second:
+        return randn(g, B, H, Tq, D, dtype=dtype, shift=shift, scale=scale), randn(g, B, H, Tk, D, dtype=dtype, shift=shift, scale=scale)
+    return randn(g, B, Tq, H, D, dtype=dtype, shift=shift, scale=scale), randn(g, B, Tk, H, D, dtype=dtype, shift=shift, scale=scale)
+
+
+# ---------------------------------------------------------------- head LayerNorm
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads_second", [True, False])
+@pytest.mark.parametrize("D", [32, 64, 96, 128, 256, 40, 59])
+@pytest.mark.parametrize("Tq,Tk", [(14, 14), (200, 200), (113, 203), (1, 239), (1024, 1023)])
+def test_head_ln(Tq, Tk, D, heads_second, dtype):
+    from rgd_triton_amd import triton_fused_ln_func_fn
+
+    g = gen(0)
+    q, k = _qk(g, 4, 9, Tq, Tk, D, dtype, heads_second, shift=0.5, scale=2.0)
+    dq_o, dk_o = _qk(g, 4, 9, Tq, Tk, D, dtype, heads_second)
+    qg, kg = to_gpu(q, k, requires_grad=True)
+    qo, ko = triton_fused_ln_func_fn(qg, kg, heads_second, 1e-6)
+    dq, dk = torch.autograd.grad((qo, ko), (qg, kg), (dq_o.to("cuda"), dk_o.to("cuda")))
+    assert_close(qo, oracle.head_ln_fwd(q), dtype, name="qo")
+    assert_close(ko, oracle.head_ln_fwd(k), dtype, name="ko")
+    assert_close(dq, oracle.head_ln_bwd(dq_o, q), dtype, name="dq")
+    assert_close(dk, oracle.head_ln_bwd(dk_o, k), dtype, name="dk")
+
+
+def test_head_ln_layout_invariance_and_views():
+    """op(x.transpose(1,2), heads_second=True) == op(x, heads_second=False).transpose(1,2), bit for bit;
+    q, k taken as views of a packed qkv buffer (token stride 3*h*d)."""
+    from rgd_triton_amd import FusedHeadLayerNorm
+
+    g = gen(1)
+    qkv = randn(g, 2, 77, 3, 6, 64, dtype=torch.bfloat16).to("cuda")
+    q, k, _ = qkv.unbind(2)  # (B,T,H,D) views, token stride 3*H*D
+    m = FusedHeadLayerNorm()
+    a_q, a_k = m(q, k, heads_second=False)
+    b_q, b_k = m(q.transpose(1, 2), k.transpose(1, 2), heads_second=True)
+    assert torch.equal(a_q, b_q.transpose(1, 2)) and torch.equal(a_k, b_k.transpose(1, 2))
+    assert_close(a_q, oracle.head_ln_fwd(q.cpu()), torch.bfloat16, name="q view")
+    c_q, _ = m(q.contiguous(), k.contiguous(), heads_second=False)
+    assert torch.equal(a_q, c_q)
+
+
+# ---------------------------------------------------------------- RoPE
+def _table(P, R, dtype, axial=False):
+    if axial:
+        L = int(P ** 0.5) + 1
+        return oracle.axial_rotary_table(L, R, 32.0, dtype)
+    return oracle.rotary_table(P, R, 10000.0, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("D,R", D_R)
+@pytest.mark.parametrize("cut", [0, 0.5, 0.75, 1.0])
+@pytest.mark.parametrize("heads_second", [True, False])
+@pytest.mark.parametrize("T", [14, 97, 384])
+def test_rope(T, heads_second, cut, D, R, dtype):
+    from rgd_triton_amd import triton_rope_fn
+
+    g = gen(0)
+    q, k = _qk(g, 4, 9, T, T, D, dtype, heads_second)
+    gq, gk = _qk(g, 4, 9, T, T, D, dtype, heads_second)
+    pe = _table(T + 1, R, dtype, axial=True)[:, : T + 1].contiguous()
+    cutoff = (int(cut * T), int(cut * T))
+    qg, kg = to_gpu(q, k, requires_grad=True)
+    qo, ko = triton_rope_fn(qg, kg, pe.to("cuda"), seq_cutoff=cutoff, heads_second=heads_second)
+    dq, dk = torch.autograd.grad((qo, ko), (qg, kg), (gq.to("cuda"), gk.to("cuda")))
+    qr, kr = oracle.rope_fwd(q, k, pe, cutoff, heads_second)
+    dqr, dkr = oracle.rope_bwd(gq, gk, pe, cutoff, heads_second)
+    for a, r, n in ((qo, qr, "qo"), (ko, kr, "ko"), (dq, dqr, "dq"), (dk, dkr, "dk")):
+        assert_close(a, r, dtype, "rope", n)
+    if cut == 0:
+        assert torch.equal(qo, qg) and torch.equal(dk.cpu(), gk)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads_second", [True, False])
+@pytest.mark.parametrize("Tq,Tk", SEQ_PAIRS)
+def test_rope_seqdiff(Tq, Tk, heads_second, dtype):
+    from rgd_triton_amd import RoPE
+
+    g = gen(2)
+    D, R = 128, 96
+    q, k = _qk(g, 3, 5, Tq, Tk, D, dtype, heads_second)
+    gq, gk = _qk(g, 3, 5, Tq, Tk, D, dtype, heads_second)
+    pe = _table(max(Tq, Tk) + 3, R, torch.float32)  # fp32 table with 16-bit q/k is allowed
+    cutoff = (int(0.75 * Tq), int(0.5 * Tk))
+    qg, kg = to_gpu(q, k, requires_grad=True)
+    qo, ko = RoPE()(qg, kg, pe.to("cuda"), seq_cutoff=cutoff, heads_second=heads_second)
+    dq, dk = torch.autograd.grad((qo, ko), (qg, kg), (gq.to("cuda"), gk.to("cuda")))
+    qr, kr = oracle.rope_fwd(q, k, pe, cutoff, heads_second)
+    dqr, dkr = oracle.rope_bwd(gq, gk, pe, cutoff, heads_second)
+    for a, r, n in ((qo, qr, "qo"), (ko, kr, "ko"), (dq, dqr, "dq"), (dk, dkr, "dk")):
+        assert_close(a, r, dtype, "rope", n)
+    assert not torch.equal(qo, qg) or cutoff[0] == 0  # out of place: the input is untouched
+    assert torch.equal(qg.detach().cpu(), q)
+
+
+def test_rope_errors_and_cutoff_forms():
+    from rgd_triton_amd import triton_rope_fn
+
+    q = torch.randn(1, 2, 16, 64, device="cuda")
+    pe = oracle.rotary_table(16, 32).to("cuda")
+    with pytest.raises(AssertionError):  # the reference requires T < P strictly
+        triton_rope_fn(q, q, pe)
+    pe = oracle.rotary_table(17, 32).to("cuda")
+    a = triton_rope_fn(q, q, pe, seq_cutoff=None)
+    b = triton_rope_fn(q, q, pe, seq_cutoff=16)
+    c = triton_rope_fn(q, q, pe, seq_cutoff=[16, 16])
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], c[1])
+    big = torch.randn(1, 2, 16, 160, device="cuda")
+    with pytest.raises(AssertionError, match="up to 128"):
+        triton_rope_fn(big, big, pe)
+    pe.requires_grad_(True)
+    qq = q.clone().requires_grad_(True)
+    out = triton_rope_fn(qq, qq, pe)
+    with pytest.raises(AssertionError, match="does not support gradients in position embeddings"):
+        torch.autograd.grad(out[0].sum(), (qq, pe))
+
+
+# ---------------------------------------------------------------- LayerNorm + RoPE
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("D,R", D_R)
+@pytest.mark.parametrize("cut", [0, 0.5, 1.0])
+@pytest.mark.parametrize("heads_second", [True, False])
+@pytest.mark.parametrize("T", [31, 200])
+def test_ln_rope(T, heads_second, cut, D, R, dtype):
+    from rgd_triton_amd import triton_fused_ln_rope_fn
+
+    g = gen(0)
+    q, k = _qk(g, 4, 9, T, T, D, dtype, heads_second, shift=0.3, scale=1.5)
+    gq, gk = _qk(g, 4, 9, T, T, D, dtype, heads_second)
+    pe = _table(T + 1, R, dtype, axial=True)[:, : T + 1].contiguous()
+    cutoff = (int(cut * T), int(cut * T))
+    qg, kg = to_gpu(q, k, requires_grad=True)
+    qo, ko = triton_fused_ln_rope_fn(qg, kg, pe.to("cuda"), seq_cutoff=cutoff, heads_second=heads_second, norm_eps=1e-6)
+    dq, dk = torch.autograd.grad((qo, ko), (qg, kg), (gq.to("cuda"), gk.to("cuda")))
+    qr, kr = oracle.ln_rope_fwd(q, k, pe, cutoff, heads_second, 1e-6)
+    dqr, dkr = oracle.ln_rope_bwd(gq, gk, q, k, pe, cutoff, heads_second, 1e-6)
+    for a, r, n in ((qo, qr, "qo"), (ko, kr, "ko"), (dq, dqr, "dq"), (dk, dkr, "dk")):
+        assert_close(a, r, dtype, "ln_rope", n)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads_second", [True, False])
+@pytest.mark.parametrize("Tq,Tk", SEQ_PAIRS)
+def test_ln_rope_seqdiff(Tq, Tk, heads_second, dtype):
+    from rgd_triton_amd import FusedLNRoPE
+
+    g = gen(4)
+    D, R = 64, 32
+    q, k = _qk(g, 3, 5, Tq, Tk, D, dtype, heads_second, shift=-0.2, scale=3.0)
+    gq, gk = _qk(g, 3, 5, Tq, Tk, D, dtype, heads_second)
+    pe = _table(max(Tq, Tk) + 1, R, dtype)
+    cutoff = (int(0.75 * Tq), Tk)
+    qg, kg = to_gpu(q, k, requires_grad=True)
+    qo, ko = FusedLNRoPE()(qg, kg, pe.to("cuda"), seq_cutoff=cutoff, heads_second=heads_second, eps=1e-5)
+    dq, dk = torch.autograd.grad((qo, ko), (qg, kg), (gq.to("cuda"), gk.to("cuda")))
+    qr, kr = oracle.ln_rope_fwd(q, k, pe, cutoff, heads_second, 1e-5)
+    dqr, dkr = oracle.ln_rope_bwd(gq, gk, q, k, pe, cutoff, heads_second, 1e-5)
+    for a, r, n in ((qo, qr, "qo"), (ko, kr, "ko"), (dq, dqr, "dq"), (dk, dkr, "dk")):
+        assert_close(a, r, dtype, "ln_rope", n)
+
+
+def test_ln_rope_equals_ln_then_rope_fp32():
+    """fusion: FusedLNRoPE == RoPE(FusedHeadLayerNorm) in fp32 within fp32 tolerance"""
+    from rgd_triton_amd import triton_fused_ln_func_fn, triton_fused_ln_rope_fn, triton_rope_fn
+
+    g = gen(5)
+    q, k = _qk(g, 2, 4, 100, 60, 96, torch.float32, False)
+    pe = oracle.rotary_table(101, 64).to("cuda")
+    qg, kg = to_gpu(q, k)
+    a = triton_fused_ln_rope_fn(qg, kg, pe, heads_second=False)
+    b = triton_rope_fn(*triton_fused_ln_func_fn(qg, kg, False), pe, heads_second=False)
+    assert_close(a[0], b[0], torch.float32, name="q")
+    assert_close(a[1], b[1], torch.float32, name="k")
+
+
+def test_ln_rope_config2_slice():
+    """BASELINE config 2 at reduced batch: q,k (2,2048,16,64) bf16, heads_second=False, eps 1e-5,
+    R=32, theta 10000, cutoff (2048,2048), P = 2049."""
+    from rgd_triton_amd import FusedLNRoPE
+
+    g = gen(1002)
+    q, k = _qk(g, 2, 16, 2048, 2048, 64, torch.bfloat16, False)
+    gq, gk = _qk(g, 2, 16, 2048, 2048, 64, torch.bfloat16, False)
+    pe = oracle.rotary_table(2049, 32, 10000.0, torch.bfloat16)
+    qg, kg = to_gpu(q, k, requires_grad=True)
+    m = FusedLNRoPE()
+    qo, ko = m(qg, kg, pe.to("cuda"), seq_cutoff=(2048, 2048), heads_second=False, eps=1e-5)
+    dq, dk = torch.autograd.grad((qo, ko), (qg, kg), (gq.to("cuda"), gk.to("cuda")))
+    qr, kr = oracle.ln_rope_fwd(q, k, pe, (2048, 2048), False, 1e-5)
+    dqr, dkr = oracle.ln_rope_bwd(gq, gk, q, k, pe, (2048, 2048), False, 1e-5)
+    for a, r, n in ((qo, qr, "qo"), (ko, kr, "ko"), (dq, dqr, "dq"), (dk, dkr, "dk")):
+        assert_close(a, r, torch.bfloat16, "ln_rope", n)
+
+
+@pytest.mark.parametrize("which", ["ln", "rope", "ln_rope"])
+def test_head_ops_deterministic(which):
+    from rgd_triton_amd import triton_fused_ln_func_fn, triton_fused_ln_rope_fn, triton_rope_fn
+
+    g = gen(6)
+    q, k = _qk(g, 60, 4, 113, 203, 64, torch.float16, True)
+    gq, gk = _qk(g, 60, 4, 113, 203, 64, torch.float16, True)
+    pe = oracle.rotary_table(204, 32, dtype=torch.float16).to("cuda")
+    qg, kg = to_gpu(q, k, requires_grad=True)
+    gq, gk = gq.cuda(), gk.cuda()
+    fn = {"ln": lambda: triton_fused_ln_func_fn(qg, kg, True),
+          "rope": lambda: triton_rope_fn(qg, kg, pe, (100, 150), True),
+          "ln_rope": lambda: triton_fused_ln_rope_fn(qg, kg, pe, (100, 150), True)}[which]
+    first = None
+    for _ in range(20):
+        out = fn()
+        gr = torch.autograd.grad(out, (qg, kg), (gq, gk))
+        cur = [t.clone() for t in (*out, *gr)]
+        if first is None:
+            first = cur
+        else:
+            assert all(torch.equal(a, b) for a, b in zip(cur, first))
