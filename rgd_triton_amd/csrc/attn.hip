@@ -1,0 +1,218 @@
+// Host side of the attention kernels: validation, dispatch and the extern "C" entry points.
+#include "attn_fwd.h"
+#include "attn_bwd.h"
+
+#include <math.h>
+#include <string.h>
+
+namespace {
+
+bool t4_vec_ok(const rgd_tensor4* t) {
+    return rgd_aligned16(t->ptr) && (t->stride_b % 8) == 0 && (t->stride_h % 8) == 0 && (t->stride_n % 8) == 0;
+}
+AttnTensor at(const rgd_tensor4* t) {
+    AttnTensor a;
+    a.ptr = t ? t->ptr : nullptr;
+    a.sb = t ? t->stride_b : 0;
+    a.sh = t ? t->stride_h : 0;
+    a.sn = t ? t->stride_n : 0;
+    return a;
+}
+
+template <typename T, int DPAD, bool HAS_BIAS> int launch_fwd(const AttnFwdParams& p, unsigned grid, hipStream_t s) {
+    auto kern = attn_fwd_kernel<T, DPAD, HAS_BIAS>;
+    constexpr size_t lds = AttnFwdSmem<DPAD>::BYTES;
+    static bool configured = false;  // benign race: the attribute is idempotent
+    if (!configured && lds > 48 * 1024) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds) != hipSuccess) {
+            rgd_set_error("rgd_attn_fwd: cannot reserve %zu bytes of LDS", lds);
+            return RGD_ERR_LAUNCH;
+        }
+        configured = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(ATTN_THREADS), lds, s, p);
+    return RGD_OK;
+}
+
+template <typename T> int dispatch_fwd(const AttnFwdParams& p, unsigned grid, hipStream_t s) {
+    const bool hb = p.bias_kind != RGD_BIAS_NONE;
+#define FWD_CASE(DP)                                                             \
+    if (p.D <= DP) return hb ? launch_fwd<T, DP, true>(p, grid, s) : launch_fwd<T, DP, false>(p, grid, s);
+    FWD_CASE(32)
+    FWD_CASE(64)
+    FWD_CASE(96)
+    FWD_CASE(128)
+#undef FWD_CASE
+    return RGD_ERR_UNSUPPORTED;
+}
+
+template <typename T, int DPAD, bool HAS_BIAS, bool DQ> int launch_bwd(const AttnBwdParams& p, unsigned grid, hipStream_t s) {
+    auto kern = DQ ? attn_bwd_dq_kernel<T, DPAD, HAS_BIAS> : attn_bwd_dkv_kernel<T, DPAD, HAS_BIAS>;
+    constexpr size_t lds = DQ ? DqSmem<DPAD>::BYTES : DkvSmem<DPAD>::BYTES;
+    static bool configured = false;
+    if (!configured && lds > 48 * 1024) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds) != hipSuccess) {
+            rgd_set_error("rgd_attn_bwd: cannot reserve %zu bytes of LDS", lds);
+            return RGD_ERR_LAUNCH;
+        }
+        configured = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(BWD_THREADS), lds, s, p);
+    return RGD_OK;
+}
+
+template <typename T, bool DQ> int dispatch_bwd(const AttnBwdParams& p, unsigned grid, hipStream_t s) {
+    const bool hb = p.bias_kind != RGD_BIAS_NONE;
+#define BWD_CASE(DP)                                                                     \
+    if (p.D <= DP) return hb ? launch_bwd<T, DP, true, DQ>(p, grid, s) : launch_bwd<T, DP, false, DQ>(p, grid, s);
+    BWD_CASE(32)
+    BWD_CASE(64)
+    BWD_CASE(96)
+    BWD_CASE(128)
+#undef BWD_CASE
+    return RGD_ERR_UNSUPPORTED;
+}
+
+int check_common(const char* name, int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, int dtype, int bias_kind,
+                 int bias_dtype, const rgd_tensor4* bias) {
+    RGD_REQUIRE(dtype == RGD_F16 || dtype == RGD_BF16, RGD_ERR_INVALID, "%s: Only support fp16 and bf16", name);
+    RGD_REQUIRE(D >= 1 && D <= 128, RGD_ERR_INVALID, "%s: FlashAttention only support head dimensions up to 128", name);
+    RGD_REQUIRE(B >= 0 && H >= 0 && Tq >= 0 && Tk >= 0, RGD_ERR_INVALID, "%s: negative shape", name);
+    RGD_REQUIRE(Tq < (1ll << 30) && Tk < (1ll << 30) && B * H < (1ll << 24), RGD_ERR_UNSUPPORTED, "%s: shape too large",
+                name);
+    RGD_REQUIRE(bias_kind == RGD_BIAS_NONE || bias_kind == RGD_BIAS_VECTOR || bias_kind == RGD_BIAS_MATRIX,
+                RGD_ERR_INVALID, "%s: bad bias kind %d", name, bias_kind);
+    if (bias_kind != RGD_BIAS_NONE) {
+        RGD_REQUIRE(bias && bias->ptr, RGD_ERR_INVALID, "%s: null bias", name);
+        RGD_REQUIRE(bias_dtype == dtype || bias_dtype == RGD_F32, RGD_ERR_INVALID,
+                    "%s: bias must have the dtype of q or fp32", name);
+    }
+    return RGD_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int64_t rgd_attn_seqlen_q_rounded(int64_t Tq) { return (Tq + 63) / 64 * 64; }
+
+int rgd_attn_fwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const rgd_tensor4* q, const rgd_tensor4* k,
+                 const rgd_tensor4* v, const rgd_tensor4* bias, int bias_kind, int bias_dtype, const rgd_tensor4* o,
+                 float* lse, int dtype, int causal, float softmax_scale, void* stream) {
+    const char* name = "rgd_attn_fwd";
+    int rc = check_common(name, B, H, Tq, Tk, D, dtype, bias_kind, bias_dtype, bias);
+    if (rc != RGD_OK) return rc;
+    if (B * H * Tq == 0) return RGD_OK;
+    RGD_REQUIRE(q && q->ptr && o && o->ptr && lse, RGD_ERR_INVALID, "%s: null tensor", name);
+    RGD_REQUIRE(Tk == 0 || (k && k->ptr && v && v->ptr), RGD_ERR_INVALID, "%s: null tensor", name);
+
+    AttnFwdParams p;
+    memset(&p, 0, sizeof(p));
+    p.q = at(q);
+    p.k = at(k);
+    p.v = at(v);
+    p.o = at(o);
+    p.lse = lse;
+    p.B = (int)B;
+    p.H = (int)H;
+    p.Tq = (int)Tq;
+    p.Tk = (int)Tk;
+    p.D = (int)D;
+    p.Tq_rounded = (int)rgd_attn_seqlen_q_rounded(Tq);
+    p.nqb = (int)((Tq + ATTN_BM - 1) / ATTN_BM);
+    p.causal = causal ? 1 : 0;
+    p.vec = (D % 8 == 0) && t4_vec_ok(q) && (Tk == 0 || (t4_vec_ok(k) && t4_vec_ok(v))) && t4_vec_ok(o);
+    p.scale_log2 = softmax_scale * kLog2e;
+    p.bias_kind = bias_kind;
+    p.bias_dtype = bias_dtype;
+    if (bias_kind != RGD_BIAS_NONE) {
+        p.bias = at(bias);
+        if (bias_kind == RGD_BIAS_VECTOR) p.bias.sn = 0;
+        const int64_t per16 = bias_dtype == RGD_F32 ? 4 : 8;  // elements per 16 bytes
+        p.bias_vec = rgd_aligned16(bias->ptr) && (p.bias.sb % per16) == 0 && (p.bias.sh % per16) == 0 &&
+                     (p.bias.sn % per16) == 0;
+    }
+    const int64_t grid = (int64_t)p.nqb * B * H;
+    RGD_REQUIRE(grid < (1ll << 31), RGD_ERR_UNSUPPORTED, "%s: grid too large", name);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    rc = dtype == RGD_F16 ? dispatch_fwd<f16_t>(p, (unsigned)grid, s) : dispatch_fwd<bf16_t>(p, (unsigned)grid, s);
+    if (rc != RGD_OK) return rc;
+    RGD_CHECK_LAUNCH(name);
+    return RGD_OK;
+}
+
+size_t rgd_attn_bwd_workspace(int64_t B, int64_t H, int64_t Tq, int64_t, int64_t) {
+    return (size_t)(B * H * rgd_attn_seqlen_q_rounded(Tq)) * sizeof(float);
+}
+
+int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const rgd_tensor4* dout, const rgd_tensor4* q,
+                 const rgd_tensor4* k, const rgd_tensor4* v, const rgd_tensor4* o, const float* lse,
+                 const rgd_tensor4* bias, int bias_kind, int bias_dtype, const rgd_tensor4* dq, const rgd_tensor4* dk,
+                 const rgd_tensor4* dv, int dtype, int causal, float softmax_scale, void* workspace,
+                 size_t workspace_bytes, void* stream) {
+    const char* name = "rgd_attn_bwd";
+    int rc = check_common(name, B, H, Tq, Tk, D, dtype, bias_kind, bias_dtype, bias);
+    if (rc != RGD_OK) return rc;
+    if (B * H == 0 || (Tq == 0 && Tk == 0)) return RGD_OK;
+    const rgd_tensor4* all[] = {dout, q, k, v, o, dq, dk, dv};
+    for (const rgd_tensor4* t : all) RGD_REQUIRE(t, RGD_ERR_INVALID, "%s: null tensor descriptor", name);
+    RGD_REQUIRE(Tq == 0 || (dout->ptr && q->ptr && o->ptr && dq->ptr && lse), RGD_ERR_INVALID, "%s: null tensor", name);
+    RGD_REQUIRE(Tk == 0 || (k->ptr && v->ptr && dk->ptr && dv->ptr), RGD_ERR_INVALID, "%s: null tensor", name);
+    RGD_REQUIRE(workspace_bytes >= rgd_attn_bwd_workspace(B, H, Tq, Tk, D) && (workspace || Tq == 0), RGD_ERR_WORKSPACE,
+                "%s: workspace too small", name);
+
+    AttnBwdParams p;
+    memset(&p, 0, sizeof(p));
+    p.q = at(q);
+    p.k = at(k);
+    p.v = at(v);
+    p.o = at(o);
+    p.dout = at(dout);
+    p.dq = at(dq);
+    p.dk = at(dk);
+    p.dv = at(dv);
+    p.lse = lse;
+    p.delta = static_cast<float*>(workspace);
+    p.B = (int)B;
+    p.H = (int)H;
+    p.Tq = (int)Tq;
+    p.Tk = (int)Tk;
+    p.D = (int)D;
+    p.Tq_rounded = (int)rgd_attn_seqlen_q_rounded(Tq);
+    p.causal = causal ? 1 : 0;
+    p.vec = (D % 8 == 0);
+    for (const rgd_tensor4* t : all) p.vec = p.vec && (t->ptr == nullptr || t4_vec_ok(t));
+    p.scale = softmax_scale;
+    p.scale_log2 = softmax_scale * kLog2e;
+    p.bias_kind = bias_kind;
+    p.bias_dtype = bias_dtype;
+    if (bias_kind != RGD_BIAS_NONE) {
+        p.bias = at(bias);
+        if (bias_kind == RGD_BIAS_VECTOR) p.bias.sn = 0;
+        const int64_t per16 = bias_dtype == RGD_F32 ? 4 : 8;
+        p.bias_vec = rgd_aligned16(bias->ptr) && (p.bias.sb % per16) == 0 && (p.bias.sh % per16) == 0 &&
+                     (p.bias.sn % per16) == 0;
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (Tq > 0) {  // dQ and delta
+        p.nblk = (int)((Tq + BWD_BM - 1) / BWD_BM);
+        const int64_t grid = (int64_t)p.nblk * B * H;
+        RGD_REQUIRE(grid < (1ll << 31), RGD_ERR_UNSUPPORTED, "%s: grid too large", name);
+        rc = dtype == RGD_F16 ? dispatch_bwd<f16_t, true>(p, (unsigned)grid, s) : dispatch_bwd<bf16_t, true>(p, (unsigned)grid, s);
+        if (rc != RGD_OK) return rc;
+        RGD_CHECK_LAUNCH(name);
+    }
+    if (Tk > 0) {  // dK and dV (reads delta)
+        p.nblk = (int)((Tk + BWD_BM - 1) / BWD_BM);
+        const int64_t grid = (int64_t)p.nblk * B * H;
+        RGD_REQUIRE(grid < (1ll << 31), RGD_ERR_UNSUPPORTED, "%s: grid too large", name);
+        rc = dtype == RGD_F16 ? dispatch_bwd<f16_t, false>(p, (unsigned)grid, s) : dispatch_bwd<bf16_t, false>(p, (unsigned)grid, s);
+        if (rc != RGD_OK) return rc;
+        RGD_CHECK_LAUNCH(name);
+    }
+    return RGD_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,268 @@
+"""GPU parity of FlashAttention / flash_attn_func against the CPU oracle.  Counterpart of the
+reference's tests/test_flash_attn.py: qkv :68-178, output :180-309, race :312-388,
+bwd_overflow :391-451, bwd_transpose :454-513.  The acceptance rule is the reference's: the error
+against the fp32 oracle may be at most a small multiple of the error of a low-precision PyTorch
+evaluation of the same formula."""
+import math
+
+import pytest
+import torch
+
+from helpers import gen, oracle, randn, to_gpu
+
+pytestmark = pytest.mark.gpu
+
+HALF = [torch.float16, torch.bfloat16]
+
+
+def make_bias(g, kind, B, H, Tq, Tk, dtype):
+    shape = {"none": None, "static": (1, 1, Tq, Tk), "batch": (B, 1, Tq, Tk), "head": (1, H, Tq, Tk),
+             "cube": (B, H, Tq, Tk), "vector": (B, H, 1, Tk)}[kind]
+    return None if shape is None else randn(g, *shape, dtype=dtype)
+
+
+def run_case(q, k, v, bias, do, causal=False, scale=None):
+    """returns (o, lse, dq, dk, dv) from the GPU and the oracle's (o, lse, dq, dk, dv) + low-precision o"""
+    from rgd_triton_amd import flash_attn_func
+
+    qg, kg, vg = to_gpu(q, k, v, requires_grad=True)
+    bg = None if bias is None else bias.to("cuda")
+    o, lse = flash_attn_func(qg, kg, vg, bg, causal, scale, return_lse=True)
+    dq, dk, dv = torch.autograd.grad(o, (qg, kg, vg), do.to("cuda"))
+    return (o, lse, dq, dk, dv)
+
+
+def reference(q, k, v, bias, do, causal=False, scale=None):
+    o_ref, lse_ref = oracle.attention_fwd(q, k, v, bias, causal, scale)
+    g_ref = oracle.attention_bwd(do, q, k, v, bias, causal, scale)
+    # the low-precision PyTorch run (upcast=False, reorder_ops=True) and its autograd gradients
+    ql, kl, vl = (t.clone().requires_grad_(True) for t in (q, k, v))
+    if scale is None:
+        o_pt = oracle.attention_lowp(ql, kl, vl, bias, causal)
+        g_pt = torch.autograd.grad(o_pt, (ql, kl, vl), do)
+    else:
+        o_pt, g_pt = None, None
+    return o_ref, lse_ref, g_ref, o_pt, g_pt
+
+
+def maxdiff(a, b):
+    return (a.detach().cpu().float() - b.detach().float()).abs().max().item()
+
+
+def check(got, ref, Tq, out_mult=2, grad_mult=2, grad_add=0.0, name=""):
+    o, lse, dq, dk, dv = got
+    o_ref, lse_ref, g_ref, o_pt, g_pt = ref
+    assert not torch.isnan(o).any() and not torch.isnan(dq).any() and not torch.isnan(dk).any() and not torch.isnan(dv).any()
+    assert maxdiff(o, o_ref) <= out_mult * maxdiff(o_pt, o_ref) + 1e-5, f"{name} o: {maxdiff(o, o_ref)} vs {maxdiff(o_pt, o_ref)}"
+    for a, r, pt, n in zip((dq, dk, dv), g_ref, g_pt, ("dq", "dk", "dv")):
+        assert maxdiff(a, r) <= grad_mult * maxdiff(pt, r) + grad_add + 1e-5, f"{name} {n}: {maxdiff(a, r)} vs {maxdiff(pt, r)}"
+    fin = torch.isfinite(lse_ref)
+    torch.testing.assert_close(lse[..., :Tq].cpu()[fin], lse_ref[fin], rtol=1e-4, atol=1e-4)
+    assert torch.all(lse[..., Tq:] == 0)
+
+
+@pytest.mark.parametrize("dtype", HALF)
+@pytest.mark.parametrize("bias_type", ["none", "static", "batch", "head", "cube"])
+@pytest.mark.parametrize("d", [32, 64])
+@pytest.mark.parametrize("seqlen", [14, 31, 97, 128, 200, 384, 768, 1025])
+def test_flash_attn_qkv(seqlen, d, bias_type, dtype):
+    """packed qkv (views with token stride 3*h*d), square attention, every bias broadcast form"""
+    g = gen(0)
+    B, H = (4, 9) if seqlen < 768 else (2, 5)
+    qkv = randn(g, 3, B, seqlen, H, d, dtype=dtype)
+    q, k, v = qkv.unbind(0)
+    bias = make_bias(g, bias_type, B, H, seqlen, seqlen, dtype)
+    do = randn(g, B, seqlen, H, d, dtype=dtype)
+    check(run_case(q, k, v, bias, do), reference(q, k, v, bias, do), seqlen, name=f"qkv {bias_type}")
+
+
+@pytest.mark.parametrize("dtype", HALF)
+@pytest.mark.parametrize("bias_type", ["none", "static", "batch", "head", "cube"])
+@pytest.mark.parametrize("d", [32, 64, 128])
+@pytest.mark.parametrize("Tq,Tk", [(113, 203), (128, 217), (113, 211), (108, 256), (256, 512), (512, 256),
+                                    (1024, 1024), (1023, 1024), (1024, 1023), (239, 1), (1, 239), (2048, 2048)])
+def test_flash_attn_output(Tq, Tk, d, bias_type, dtype):
+    if Tq == 2048 and (bias_type not in ("none", "cube") or d == 32):
+        pytest.skip("large case kept for two bias forms")
+    g = gen(0)
+    # the CPU oracle dominates the run time: fewer (batch, head) pairs for the long sequences
+    B, H = (2, 3) if Tq >= 1023 else (4, 9)
+    q, k, v = randn(g, B, Tq, H, d, dtype=dtype), randn(g, B, Tk, H, d, dtype=dtype), randn(g, B, Tk, H, d, dtype=dtype)
+    bias = make_bias(g, bias_type, B, H, Tq, Tk, dtype)
+    do = randn(g, B, Tq, H, d, dtype=dtype)
+    check(run_case(q, k, v, bias, do), reference(q, k, v, bias, do), Tq, grad_mult=3, name=f"out {bias_type}")
+
+
+@pytest.mark.parametrize("dtype", HALF)
+@pytest.mark.parametrize("d", [40, 59, 80, 96, 111, 128, 8, 16])
+@pytest.mark.parametrize("Tq,Tk", [(97, 131), (256, 128)])
+def test_flash_attn_head_dims(Tq, Tk, d, dtype):
+    """head dims that are not powers of two, including ones whose rows are not 16-byte aligned"""
+    g = gen(1)
+    q, k, v = randn(g, 2, Tq, 3, d, dtype=dtype), randn(g, 2, Tk, 3, d, dtype=dtype), randn(g, 2, Tk, 3, d, dtype=dtype)
+    bias = make_bias(g, "cube", 2, 3, Tq, Tk, dtype)
+    do = randn(g, 2, Tq, 3, d, dtype=dtype)
+    check(run_case(q, k, v, bias, do), reference(q, k, v, bias, do), Tq, grad_mult=3, name=f"d={d}")
+
+
+@pytest.mark.parametrize("dtype", HALF)
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("bias_type", ["none", "vector", "cube"])
+@pytest.mark.parametrize("Tq,Tk", [(128, 128), (200, 200), (113, 203), (300, 150), (1, 64)])
+def test_flash_attn_causal_vector_fp32bias(Tq, Tk, bias_type, causal, dtype):
+    """API corners the reference implements but does not test: causal (top-left aligned), vector bias
+    (.., 1, Tk), fp32 bias with 16-bit q"""
+    g = gen(2)
+    B, H, d = 2, 4, 64
+    q, k, v = randn(g, B, Tq, H, d, dtype=dtype), randn(g, B, Tk, H, d, dtype=dtype), randn(g, B, Tk, H, d, dtype=dtype)
+    bias = make_bias(g, bias_type, B, H, Tq, Tk, torch.float32)
+    do = randn(g, B, Tq, H, d, dtype=dtype)
+    # the low-precision comparison run adds the bias in q's dtype
+    ref = reference(q, k, v, bias, do, causal)
+    if bias is not None:
+        ref_lp = reference(q, k, v, bias.to(dtype), do, causal)
+        ref = ref[:3] + ref_lp[3:]
+    check(run_case(q, k, v, bias, do, causal), ref, Tq, grad_mult=3, grad_add=2e-3, name=f"causal={causal} {bias_type}")
+
+
+@pytest.mark.parametrize("dtype", HALF)
+def test_flash_attn_softmax_scale_and_lse(dtype):
+    g = gen(3)
+    q, k, v = randn(g, 2, 150, 4, 64, dtype=dtype), randn(g, 2, 90, 4, 64, dtype=dtype), randn(g, 2, 90, 4, 64, dtype=dtype)
+    do = randn(g, 2, 150, 4, 64, dtype=dtype)
+    got = run_case(q, k, v, None, do, scale=0.2)
+    o_ref, lse_ref, g_ref, _, _ = reference(q, k, v, None, do, scale=0.2)
+    tol = 2e-2 if dtype == torch.bfloat16 else 3e-3
+    assert maxdiff(got[0], o_ref) <= tol
+    torch.testing.assert_close(got[1][..., :150].cpu(), lse_ref, rtol=1e-4, atol=1e-4)
+    for a, r in zip(got[2:], g_ref):
+        assert maxdiff(a, r) <= 4 * tol
+    assert got[1].shape == (2, 4, 192)
+
+
+@pytest.mark.parametrize("dtype", HALF)
+@pytest.mark.parametrize("seqlen", [1, 2, 5, 17, 128])
+def test_flash_attn_bwd_overflow(seqlen, dtype):
+    """large-magnitude inputs (q x5, k and v x3), tests/test_flash_attn.py:391-451"""
+    g = gen(4)
+    B, H, d = 2, 5, 64
+    q = randn(g, B, seqlen, H, d, dtype=dtype, scale=5.0)
+    k, v = randn(g, B, seqlen, H, d, dtype=dtype, scale=3.0), randn(g, B, seqlen, H, d, dtype=dtype, scale=3.0)
+    do = randn(g, B, seqlen, H, d, dtype=dtype)
+    check(run_case(q, k, v, None, do), reference(q, k, v, None, do), seqlen, grad_mult=5, grad_add=1e-3, name="overflow")
+
+
+@pytest.mark.parametrize("dtype", HALF)
+@pytest.mark.parametrize("Tq,Tk", [(128, 128), (113, 203), (256, 512), (1, 239)])
+def test_flash_attn_bwd_transpose(Tq, Tk, dtype):
+    """non-contiguous upstream gradient and heads-first storage of q, k, v (tests/test_flash_attn.py:454-513)"""
+    from rgd_triton_amd import flash_attn_func
+
+    g = gen(5)
+    B, H, d = 3, 4, 64
+    q = randn(g, B, H, Tq, d, dtype=dtype).transpose(1, 2)
+    k, v = randn(g, B, H, Tk, d, dtype=dtype).transpose(1, 2), randn(g, B, H, Tk, d, dtype=dtype).transpose(1, 2)
+    do = randn(g, B, H, Tq, d, dtype=dtype).transpose(1, 2)
+    qg = q.transpose(1, 2).contiguous().to("cuda").transpose(1, 2).requires_grad_(True)
+    kg = k.transpose(1, 2).contiguous().to("cuda").transpose(1, 2).requires_grad_(True)
+    vg = v.transpose(1, 2).contiguous().to("cuda").transpose(1, 2).requires_grad_(True)
+    dog = do.transpose(1, 2).contiguous().to("cuda").transpose(1, 2)
+    assert Tq == 1 or (not qg.is_contiguous() and not dog.is_contiguous())
+    o, lse = flash_attn_func(qg, kg, vg, None, False, None, return_lse=True)
+    dq, dk, dv = torch.autograd.grad(o, (qg, kg, vg), dog)
+    check((o, lse, dq, dk, dv), reference(q, k, v, None, do), Tq, name="transpose")
+
+
+def test_flash_attn_masked_bias_no_nan():
+    """-inf in the bias: block-causal mask (blocks of 128, as BASELINE config 4) and padded keys
+    (as config 5).  dk/dv rows of fully masked keys are exactly zero; nothing is NaN."""
+    g = gen(6)
+    B, H, T, d = 2, 3, 384, 64
+    dtype = torch.float16
+    q, k, v = randn(g, B, T, H, d, dtype=dtype), randn(g, B, T, H, d, dtype=dtype), randn(g, B, T, H, d, dtype=dtype)
+    do = randn(g, B, T, H, d, dtype=dtype)
+    bias = (0.5 * torch.randn(B, H, T, T, generator=g)).to(dtype)
+    i = torch.arange(T)
+    bias.masked_fill_((i[None, :] // 128) > (i[:, None] // 128), float("-inf"))
+    check(run_case(q, k, v, bias, do), reference(q, k, v, bias, do), T, grad_mult=3, name="block causal")
+    pad = torch.zeros(B, 1, T, T)
+    dead = torch.randperm(T, generator=g)[:40]
+    pad[:, :, :, dead] = float("-inf")
+    pad = pad.to(torch.bfloat16)
+    qb, kb, vb, dob = (t.to(torch.bfloat16) for t in (q, k, v, do))
+    got = run_case(qb, kb, vb, pad, dob)
+    check(got, reference(qb, kb, vb, pad, dob), T, grad_mult=3, name="padded keys")
+    assert torch.all(got[3][:, dead] == 0) and torch.all(got[4][:, dead] == 0)
+    # a first key tile that is entirely -inf must not poison the running max
+    first = torch.zeros(1, 1, T, T)
+    first[..., :128] = float("-inf")
+    got = run_case(qb, kb, vb, first.to(torch.bfloat16), dob)
+    check(got, reference(qb, kb, vb, first.to(torch.bfloat16), dob), T, grad_mult=3, name="first tile masked")
+
+
+def test_flash_attn_fully_masked_row_gives_zero():
+    g = gen(7)
+    q, k, v = (randn(g, 1, 70, 2, 32, dtype=torch.float16) for _ in range(3))
+    bias = torch.zeros(1, 1, 70, 70, dtype=torch.float16)
+    bias[0, 0, 5, :] = float("-inf")
+    do = randn(g, 1, 70, 2, 32, dtype=torch.float16)
+    o, lse, dq, dk, dv = run_case(q, k, v, bias, do)
+    assert torch.all(o[0, 5] == 0) and torch.all(torch.isinf(lse[0, :, 5])) and torch.all(dq[0, 5] == 0)
+    for t in (o, dq, dk, dv):
+        assert not torch.isnan(t).any()
+
+
+@pytest.mark.parametrize("d", [32, 64])
+@pytest.mark.parametrize("bias_type", ["none", "cube"])
+@pytest.mark.parametrize("Tq,Tk", [(113, 203), (128, 217), (256, 512), (1023, 1024), (1, 239), (239, 1)])
+def test_flash_attn_race_condition(Tq, Tk, bias_type, d):
+    """The reference's determinism test (tests/test_flash_attn.py:312-388): batch 60, repeated
+    forward+backward must reproduce o, lse, dq, dk, dv bit for bit."""
+    from rgd_triton_amd import flash_attn_func
+
+    g = gen(8)
+    dtype = torch.float16
+    B, H = 60, 4
+    q, k, v = randn(g, B, Tq, H, d, dtype=dtype), randn(g, B, Tk, H, d, dtype=dtype), randn(g, B, Tk, H, d, dtype=dtype)
+    bias = make_bias(g, bias_type, B, H, Tq, Tk, dtype)
+    do = randn(g, B, Tq, H, d, dtype=dtype).to("cuda")
+    qg, kg, vg = to_gpu(q, k, v, requires_grad=True)
+    bg = None if bias is None else bias.to("cuda")
+    first = None
+    for _ in range(20):
+        o, lse = flash_attn_func(qg, kg, vg, bg, False, None, return_lse=True)
+        grads = torch.autograd.grad(o, (qg, kg, vg), do)
+        cur = [t.clone() for t in (o, lse, *grads)]
+        if first is None:
+            first = cur
+        else:
+            for a, b_, n in zip(cur, first, ("o", "lse", "dq", "dk", "dv")):
+                assert torch.equal(a, b_), f"{n} differs between runs"
+
+
+def test_flash_attn_module_errors_and_cache():
+    from rgd_triton_amd import FlashAttention, flash_attn_func
+
+    m = FlashAttention()
+    assert m.cache.fwd is None and m.cache.bwd is None and m.cache.bwd_odot is None
+    q = torch.randn(1, 64, 2, 64, device="cuda", dtype=torch.float16, requires_grad=True)
+    o = m(q, q, q)
+    o.sum().backward()
+    assert m.cache.fwd is not None and m.cache.bwd is not None and m.cache.bwd_odot is not None
+    # a different shape and bias kind through the same cache must not reuse anything stale
+    q2 = torch.randn(2, 100, 2, 32, device="cuda", dtype=torch.float16)
+    b2 = torch.randn(2, 2, 100, 100, device="cuda", dtype=torch.float16)
+    o2 = m(q2, q2, q2, bias=b2)
+    o2_ref, _ = oracle.attention_fwd(q2.cpu(), q2.cpu(), q2.cpu(), b2.cpu())
+    assert maxdiff(o2, o2_ref) < 5e-3
+    with pytest.raises(AssertionError, match="Only support fp16 and bf16"):
+        flash_attn_func(q.float(), q.float(), q.float())
+    big = torch.randn(1, 8, 1, 256, device="cuda", dtype=torch.float16)
+    with pytest.raises(AssertionError, match="head dimensions up to 128"):
+        flash_attn_func(big, big, big)
+    with pytest.raises(RuntimeError, match="Last 2 dimensions of bias"):
+        flash_attn_func(q, q, q, torch.zeros(1, 1, 3, 64, device="cuda", dtype=torch.float16))
+    bias = torch.zeros(1, 1, 64, 64, device="cuda", dtype=torch.float16, requires_grad=True)
+    out = flash_attn_func(q, q, q, bias)
+    with pytest.raises(AssertionError, match="does not support bias gradient"):
+        out.sum().backward()
