@@ -116,6 +116,45 @@ __device__ __forceinline__ void store_chunk(T* __restrict__ p, int first, int li
     }
 }
 
+// Branch-free variant used in the streaming loops: the load is unconditional (a chunk that is out of
+// range reads the start of the row instead, which is always valid memory) and out-of-range elements are
+// zeroed by a select when the raw bits are decoded.  Issue every load() of an iteration first, then
+// decode(): the loads overlap and the wavefront waits once.
+template <typename T, int N, bool VECTOR> struct Chunk {
+    static constexpr bool VEC = VECTOR && (N * sizeof(T)) % 16 == 0;
+    static constexpr int NVEC = VEC ? (N * sizeof(T)) / 16 : 1;
+    static constexpr int EPV = 16 / sizeof(T);
+    u32x4 v[NVEC];
+    T s[VEC ? 1 : N];
+
+    __device__ __forceinline__ void load(const T* __restrict__ row, int first, int limit) {
+        if constexpr (VEC) {
+            const u32x4* p = reinterpret_cast<const u32x4*>(row + (first < limit ? first : 0));
+#pragma unroll
+            for (int i = 0; i < NVEC; ++i) v[i] = p[i];
+        } else {
+#pragma unroll
+            for (int e = 0; e < N; ++e) s[e] = row[first + e < limit ? first + e : 0];
+        }
+    }
+    // MASK = false skips the zeroing selects (the caller knows every element is in range)
+    template <bool MASK = true> __device__ __forceinline__ void decode(int first, int limit, float (&out)[N]) const {
+        if constexpr (VEC) {
+            const bool ok = !MASK || first < limit;
+#pragma unroll
+            for (int i = 0; i < NVEC; ++i) {
+                T tmp[EPV];
+                __builtin_memcpy(tmp, &v[i], 16);
+#pragma unroll
+                for (int e = 0; e < EPV; ++e) out[i * EPV + e] = ok ? to_f32<T>(tmp[e]) : 0.f;
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < N; ++e) out[e] = (!MASK || first + e < limit) ? to_f32<T>(s[e]) : 0.f;
+        }
+    }
+};
+
 // chunk load whose element type is only known at run time (weights, rotary tables)
 template <int N, bool VECTOR>
 __device__ __forceinline__ void load_chunk_dyn(const void* p, int dtype, int first, int limit, float (&out)[N]) {

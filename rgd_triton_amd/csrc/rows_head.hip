@@ -81,32 +81,43 @@ int head_launch(const char* name, int mode, int64_t B, int64_t H, int64_t Tq, in
         h.token_is_inner = token_inner ? 1 : 0;
         h.cutoff = 0;
     }
-    p.total_rows = p.h[0].rows + p.h[1].rows;
     p.D = (int)D;
     p.inv_d = 1.0f / (float)D;
     p.eps = eps;
+    HeadConfig cfg;
+    cfg.mode = mode;
+    cfg.table_f32 = false;
     if (rope) {
         RGD_REQUIRE(rope->pe && rgd_dtype_ok(rope->dtype), RGD_ERR_INVALID, "%s: bad pos_emb", name);
+        RGD_REQUIRE(rope->dtype == dtype || rope->dtype == RGD_F32, RGD_ERR_UNSUPPORTED,
+                    "%s: pos_emb must have the dtype of the tensors or fp32", name);
         RGD_REQUIRE(rope->R >= 0 && rope->R <= D, RGD_ERR_INVALID, "%s: rotary dim %lld exceeds head dim %lld", name,
                     (long long)rope->R, (long long)D);
         RGD_REQUIRE(Tq < rope->P && Tk < rope->P, RGD_ERR_INVALID,
                     "%s: sequence length must be smaller than the pos_emb length %lld", name, (long long)rope->P);
         const int ps = rgd_dtype_size(rope->dtype);
+        cfg.table_f32 = rope->dtype == RGD_F32 && dtype != RGD_F32;
         p.pe = rope->pe;
         p.pe_ss = rope->ss;
         p.pe_sn = rope->sn;
-        p.pe_dtype = rope->dtype;
         p.R = (int)rope->R;
         p.rope_bwd = rope->bwd;
         p.h[0].cutoff = (int)std::max<int64_t>(0, std::min<int64_t>(rope->q_cutoff, Tq));
         p.h[1].cutoff = (int)std::max<int64_t>(0, std::min<int64_t>(rope->k_cutoff, Tk));
-        const int vec = vector ? 16 / es : 2;
-        p.pe_vec = rgd_aligned16(rope->pe) && (rope->ss * ps) % 16 == 0 && (rope->sn * ps) % 16 == 0 &&
-                   (rope->R % vec) == 0 && (vec * ps) % 16 == 0;
+        if (rope->R == 0) {
+            // nothing to rotate: the kernel still reads a table chunk per row and discards it, so point
+            // the table at memory that certainly exists
+            p.pe = xs[p.h[0].rows ? 0 : 1]->ptr;
+            p.pe_ss = p.pe_sn = 0;
+            cfg.table_f32 = false;
+        } else {
+            // the table is read with the same access width as the tensors
+            const int vec_elems = 16 / es;
+            vector = vector && rgd_aligned16(rope->pe) && (rope->ss * ps) % 16 == 0 && (rope->sn * ps) % 16 == 0 &&
+                     (rope->R % vec_elems) == 0;
+        }
     }
 
-    HeadConfig cfg;
-    cfg.mode = mode;
     cfg.vector = vector;
     const int vec = vector ? 16 / es : 2;
     const int chunks = (int)((D + vec - 1) / vec);
@@ -119,7 +130,8 @@ int head_launch(const char* name, int mode, int64_t B, int64_t H, int64_t Tq, in
         RGD_REQUIRE(chunks <= 128, RGD_ERR_UNSUPPORTED, "%s: head dim too large", name);
     }
     const int rows_per_block = 4 * (64 / cfg.G) * head_unroll(mode, cfg.NV);
-    const int64_t blocks = ((int64_t)p.total_rows + rows_per_block - 1) / rows_per_block;
+    p.blocks_q = (uint32_t)(((int64_t)p.h[0].rows + rows_per_block - 1) / rows_per_block);
+    const int64_t blocks = p.blocks_q + ((int64_t)p.h[1].rows + rows_per_block - 1) / rows_per_block;
     const dim3 grid((unsigned)blocks, 1, 1);
     hipStream_t s = static_cast<hipStream_t>(stream);
     int rc;
