@@ -11,7 +11,8 @@ import threading
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "librgd_hip.so")
+# RGD_HIP_LIB overrides the library path (used to compare kernel build variants)
+LIB_PATH = os.environ.get("RGD_HIP_LIB") or os.path.join(_HERE, "librgd_hip.so")
 HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "rgd_hip.h")
 
 RGD_F32, RGD_F16, RGD_BF16 = 0, 1, 2

@@ -3,6 +3,7 @@
 #include "attn_bwd.h"
 
 #include <math.h>
+#include <stdlib.h>
 #include <string.h>
 
 namespace {
@@ -107,6 +108,10 @@ int rgd_attn_fwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
     if (B * H * Tq == 0) return RGD_OK;
     RGD_REQUIRE(q && q->ptr && o && o->ptr && lse, RGD_ERR_INVALID, "%s: null tensor", name);
     RGD_REQUIRE(Tk == 0 || (k && k->ptr && v && v->ptr), RGD_ERR_INVALID, "%s: null tensor", name);
+
+    // offsets inside one K/V tile are kept in 32 bits
+    RGD_REQUIRE(Tk == 0 || (llabs(k->stride_n) < (1ll << 24) && llabs(v->stride_n) < (1ll << 24)), RGD_ERR_UNSUPPORTED,
+                "%s: key/value token stride too large", name);
 
     AttnFwdParams p;
     memset(&p, 0, sizeof(p));

@@ -34,31 +34,6 @@ struct AttnBwdParams {
     float scale, scale_log2;
 };
 
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-
-// 4 elements for this lane out of a transposing read; `p` is this lane's own 8-byte source piece
-template <typename T> __device__ __forceinline__ u32x2 lds_read_tr(const T* p) {
-    s16x4 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p));
-    return __builtin_bit_cast(u32x2, r);
-}
-
-// A operand (32 rows x 16 k) taken transposed from a row-major tile: MFMA row r = matrix COLUMN
-// col0 + perm(r), k index = tile ROW.  `row0` is the first of this lane-half's 8 tile rows.
-// lane decomposition: s = lane%16 -> (j = s/4 tile row within a group of 4, c = s%4 column quad),
-// gi = (lane/16)%2 selects MFMA rows 16..31.
-template <typename T>
-__device__ __forceinline__ typename Mfma<T>::V8 load_a_transposed(const T* tile, int stride, int row0, int col0,
-                                                                   int lane) {
-    const int s = lane & 15;
-    const int j = s >> 2;
-    const int cq = mfma_row_perm(((lane >> 4) & 1) * 16 + (s & 3) * 4);
-    const T* p = tile + (row0 + j) * stride + col0 + cq;
-    const u32x2 lo = lds_read_tr<T>(p);
-    const u32x2 hi = lds_read_tr<T>(p + 4 * stride);
-    const u32x4 raw = {lo[0], lo[1], hi[0], hi[1]};
-    return as_v8<T>(raw);
-}
-
 template <int DPAD> struct BwdTile {
     static constexpr int S = DPAD + 8;  // row stride of every staged tile (elements)
 };

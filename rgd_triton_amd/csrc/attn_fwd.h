@@ -4,13 +4,21 @@
 // rows and walks the keys in tiles of 64.  Everything is computed transposed so that a query row
 // lives in ONE lane column (lane % 32) for both matrix products:
 //     S^T (keys x queries) = K (keys x d) . Q^T (d x queries)      A = K tile from LDS, B = Q in registers
-//     O^T (d x queries)   += V^T (d x keys) . P^T (keys x queries)  A = V^T tile from LDS, B = P in registers
+//     O^T (d x queries)   += V^T (d x keys) . P^T (keys x queries)  A = V^T from LDS,    B = P in registers
 // The accumulator layout of S^T is exactly the B-operand layout of the second product, so the
-// probabilities never leave registers, the online-softmax state (running max, running sum) is one
-// value per lane, and the row reductions are 31 in-lane ops plus one exchange with lane ^ 32.
-// K (row-major) and V (transposed on the way in) are staged through double-buffered LDS tiles;
-// global loads of tile j+1 are in flight while tile j is in the matrix cores.  The bias tile is read
-// straight from HBM as 16-element contiguous runs per lane (32 or 64 bytes) and is touched once.
+// probabilities never leave registers, the softmax state (reference exponent, running sum) is one
+// value per lane, and a row reduction is in-lane work plus one exchange with lane ^ 32.
+//
+// K and V tiles are stored row-major in double-buffered LDS exactly as they arrive from HBM (16-byte
+// stores); V^T operands are fetched with transposing LDS reads.  Global loads of tile j+1 are in
+// flight while tile j is in the matrix cores.  The bias tile is read straight from HBM as 16-element
+// contiguous runs per lane and is touched once.
+//
+// Softmax arithmetic (log2 domain, c = scale*log2e): t = s*c + bias*log2e - m is formed with fused
+// multiply-adds against the running reference exponent m; m only moves when some logit exceeds it by
+// more than 2^8 (then the accumulators are rescaled), so the usual per-tile subtract/rescale pass is
+// rare after the first tiles.  p = exp2(t) <= 256 is safe for fp16/bf16 operands and fp32 sums, and
+// LSE = (m + log2(l)) * ln2 does not depend on where m sits.
 #pragma once
 
 #include "attn_common.h"
@@ -18,6 +26,7 @@
 constexpr int ATTN_BM = 128;  // query rows per workgroup
 constexpr int ATTN_BN = 64;   // keys per tile
 constexpr int ATTN_THREADS = 256;
+constexpr float ATTN_RESCALE_THRESHOLD = 8.0f;  // log2 units
 
 struct AttnFwdParams {
     AttnTensor q, k, v, bias, o;
@@ -28,27 +37,24 @@ struct AttnFwdParams {
 };
 
 template <int DPAD> struct AttnFwdSmem {
-    static constexpr int KS = DPAD + 8;     // K tile row stride (elements)
-    static constexpr int VS = ATTN_BN + 8;  // V^T tile row stride (elements)
-    static constexpr int K_ELEMS = ATTN_BN * KS;
-    static constexpr int V_ELEMS = DPAD * VS;
-    static constexpr size_t BYTES = 2 * (K_ELEMS + V_ELEMS) * 2;
+    static constexpr int ST = DPAD + 8;  // row stride of the K and V tiles (elements)
+    static constexpr int TILE = ATTN_BN * ST;
+    static constexpr size_t BYTES = 2 * 2 * TILE * 2;  // K and V, double buffered
 };
 
 template <typename T, int DPAD, bool HAS_BIAS>
-__global__ __launch_bounds__(ATTN_THREADS) void attn_fwd_kernel(const AttnFwdParams p) {
+__global__ __launch_bounds__(ATTN_THREADS, DPAD <= 64 ? 2 : 1) void attn_fwd_kernel(const AttnFwdParams p) {
     typedef Mfma<T> MM;
     typedef AttnFwdSmem<DPAD> SM;
+    constexpr int ST = SM::ST;
+    constexpr int TILE = SM::TILE;
     constexpr int NC = DPAD / 16;   // d chunks of the first product
     constexpr int NDB = DPAD / 32;  // 32-row blocks of O^T
     constexpr int CPR = DPAD / 8;   // 16-byte chunks per K/V row
-    constexpr int K_LOADS = ATTN_BN * CPR / ATTN_THREADS;        // per thread, per tile
-    constexpr int V_TASKS = (ATTN_BN / 2) * CPR;  // (key pair, chunk) items per tile
-    constexpr int V_LOADS = (V_TASKS + ATTN_THREADS - 1) / ATTN_THREADS;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     T* const ks_base = reinterpret_cast<T*>(smem_raw);
-    T* const vt_base = ks_base + 2 * SM::K_ELEMS;
+    T* const vs_base = ks_base + 2 * TILE;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -66,8 +72,6 @@ __global__ __launch_bounds__(ATTN_THREADS) void attn_fwd_kernel(const AttnFwdPar
     const int q_ld = q_valid ? q_row : p.Tq - 1;
 
     const T* qp = static_cast<const T*>(p.q.ptr) + b * p.q.sb + h * p.q.sh + (int64_t)q_ld * p.q.sn;
-    const T* kp = static_cast<const T*>(p.k.ptr) + b * p.k.sb + h * p.k.sh;
-    const T* vp = static_cast<const T*>(p.v.ptr) + b * p.v.sb + h * p.v.sh;
     const bool vec = p.vec != 0;
 
     typename MM::V8 qreg[NC];
@@ -79,59 +83,55 @@ __global__ __launch_bounds__(ATTN_THREADS) void attn_fwd_kernel(const AttnFwdPar
     for (int d = 0; d < NDB; ++d)
 #pragma unroll
         for (int v = 0; v < 16; ++v) oacc[d][v] = 0.f;
-    float m_run = -INFINITY;  // running max of the scaled logits (log2 domain)
-    float l_run = 0.f;        // running sum over this lane's keys
+    float m_ref = -INFINITY;  // reference exponent of this row (log2 domain); -inf until a finite logit is seen
+    float l_run = 0.f;        // sum of p over this lane's keys, relative to m_ref
 
     int ntiles = (p.Tk + ATTN_BN - 1) / ATTN_BN;
     if (p.causal) ntiles = min(ntiles, (min(p.Tq, (qb + 1) * ATTN_BM) + ATTN_BN - 1) / ATTN_BN);
 
-    u32x4 kst[K_LOADS];
-    u32x4 vst[V_LOADS][2];
-
+    // global -> register staging of the next tile.  Thread t moves the 16-byte chunks t, t+256, ... of the
+    // tile; its offsets inside a tile are fixed, the tile base is wavefront-uniform.
+    constexpr int TASKS = ATTN_BN * CPR;
+    static_assert(TASKS % ATTN_THREADS == 0, "tile chunks must divide evenly over the workgroup");
+    constexpr int LOADS = TASKS / ATTN_THREADS;
+    const T* kbase = static_cast<const T*>(p.k.ptr) + b * p.k.sb + h * p.k.sh;
+    const T* vbase = static_cast<const T*>(p.v.ptr) + b * p.v.sb + h * p.v.sh;
+    int ld_key[LOADS], ld_dc[LOADS], koff[LOADS], voff[LOADS], soff[LOADS];
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+        const int id = tid + i * ATTN_THREADS;
+        ld_key[i] = id / CPR;
+        ld_dc[i] = id % CPR;
+        koff[i] = ld_key[i] * (int)p.k.sn + ld_dc[i] * 8;
+        voff[i] = ld_key[i] * (int)p.v.sn + ld_dc[i] * 8;
+        soff[i] = ld_key[i] * ST + ld_dc[i] * 8;
+    }
+    const bool fast_tiles = vec && p.D == DPAD;  // full rows, 16-byte loads: no masking except in the last tile
+    u32x4 kst[LOADS], vst[LOADS];
     auto issue_loads = [&](int tile) {
         const int key0 = tile * ATTN_BN;
+        const T* kt = kbase + (int64_t)key0 * p.k.sn;
+        const T* vt = vbase + (int64_t)key0 * p.v.sn;
+        if (fast_tiles && key0 + ATTN_BN <= p.Tk) {
 #pragma unroll
-        for (int i = 0; i < K_LOADS; ++i) {
-            const int id = tid + i * ATTN_THREADS;
-            const int key = id / CPR, dc = id % CPR;
-            kst[i] = load8<T>(kp + (int64_t)(key0 + key) * p.k.sn, dc * 8, p.D, key0 + key < p.Tk, vec);
-        }
+            for (int i = 0; i < LOADS; ++i) {
+                kst[i] = *reinterpret_cast<const u32x4*>(kt + koff[i]);
+                vst[i] = *reinterpret_cast<const u32x4*>(vt + voff[i]);
+            }
+        } else {
 #pragma unroll
-        for (int i = 0; i < V_LOADS; ++i) {
-            const int id = tid + i * ATTN_THREADS;
-            const int kpair = id / CPR, dc = id % CPR;
-            const int key = key0 + 2 * kpair;
-            const bool live = id < V_TASKS;
-            vst[i][0] = load8<T>(vp + (int64_t)key * p.v.sn, dc * 8, p.D, live && key < p.Tk, vec);
-            vst[i][1] = load8<T>(vp + (int64_t)(key + 1) * p.v.sn, dc * 8, p.D, live && key + 1 < p.Tk, vec);
+            for (int i = 0; i < LOADS; ++i) {
+                const bool ok = key0 + ld_key[i] < p.Tk;
+                kst[i] = load8<T>(kt + (int64_t)ld_key[i] * p.k.sn, ld_dc[i] * 8, p.D, ok, vec);
+                vst[i] = load8<T>(vt + (int64_t)ld_key[i] * p.v.sn, ld_dc[i] * 8, p.D, ok, vec);
+            }
         }
     };
     auto store_tiles = [&](int buf) {
-        T* ks = ks_base + buf * SM::K_ELEMS;
-        T* vt = vt_base + buf * SM::V_ELEMS;
 #pragma unroll
-        for (int i = 0; i < K_LOADS; ++i) {
-            const int id = tid + i * ATTN_THREADS;
-            const int key = id / CPR, dc = id % CPR;
-            *reinterpret_cast<u32x4*>(ks + key * SM::KS + dc * 8) = kst[i];
-        }
-#pragma unroll
-        for (int i = 0; i < V_LOADS; ++i) {
-            const int id = tid + i * ATTN_THREADS;
-            const int kpair = id / CPR, dc = id % CPR;
-            if (id >= V_TASKS) continue;
-            Pack16 a, c;
-            a.v = vst[i][0];
-            c.v = vst[i][1];
-            uint32_t* vt32 = reinterpret_cast<uint32_t*>(vt);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                // (key, d) and (key+1, d) side by side in row d of the transposed tile
-                const uint32_t lo = __builtin_amdgcn_perm(c.w[e], a.w[e], 0x05040100);  // low halves
-                const uint32_t hi = __builtin_amdgcn_perm(c.w[e], a.w[e], 0x07060302);  // high halves
-                vt32[((dc * 8 + 2 * e) * SM::VS) / 2 + kpair] = lo;
-                vt32[((dc * 8 + 2 * e + 1) * SM::VS) / 2 + kpair] = hi;
-            }
+        for (int i = 0; i < LOADS; ++i) {
+            *reinterpret_cast<u32x4*>(ks_base + buf * TILE + soff[i]) = kst[i];
+            *reinterpret_cast<u32x4*>(vs_base + buf * TILE + soff[i]) = vst[i];
         }
     };
 
@@ -141,7 +141,11 @@ __global__ __launch_bounds__(ATTN_THREADS) void attn_fwd_kernel(const AttnFwdPar
     }
     __syncthreads();
 
-    const int krow = mfma_row_perm(li);  // matrix row this lane reads for an A operand
+    // per-lane LDS offsets (elements) of the operand reads; everything else is a compile-time offset
+    const int a_off = mfma_row_perm(li) * ST + g * 8;  // K rows as A operand
+    const int tr_off = ((lane & 15) >> 2) * ST + mfma_row_perm(((lane >> 4) & 1) * 16 + (lane & 3) * 4) +
+                       g * 16 * ST;  // V^T via transposing reads: tile row (key) j, column quad
+
     const char* bias_base = nullptr;
     int64_t bias_row = 0;
     if constexpr (HAS_BIAS) {
@@ -159,12 +163,12 @@ __global__ __launch_bounds__(ATTN_THREADS) void attn_fwd_kernel(const AttnFwdPar
         if constexpr (HAS_BIAS) {
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
-                load_bias16(bias_base, bias_row, p.bias_dtype, key0 + kb * 32 + g * 16, p.Tk, p.bias_vec && !tail, kLog2e,
+                load_bias16(bias_base, bias_row, p.bias_dtype, key0 + kb * 32 + g * 16, p.Tk, p.bias_vec && !tail, 1.0f,
                             bias_v[kb]);
         }
 
         // ---- S^T = K . Q^T ----
-        const T* ks = ks_base + buf * SM::K_ELEMS;
+        const T* ks = ks_base + buf * TILE + a_off;
         f32x16 s[2];
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
@@ -172,51 +176,73 @@ __global__ __launch_bounds__(ATTN_THREADS) void attn_fwd_kernel(const AttnFwdPar
             for (int v = 0; v < 16; ++v) s[kb][v] = 0.f;
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
-                const u32x4 a = *reinterpret_cast<const u32x4*>(ks + (kb * 32 + krow) * SM::KS + c * 16 + g * 8);
+                const u32x4 a = *reinterpret_cast<const u32x4*>(ks + kb * 32 * ST + c * 16);
                 s[kb] = MM::run(as_v8<T>(a), qreg[c], s[kb]);
             }
         }
 
-        // ---- logits in the log2 domain, masks ----
-        const bool diag = p.causal && (key0 + ATTN_BN - 1 > qb * ATTN_BM + wave * 32);
-        float mt = -INFINITY;
+        // ---- t = logit - m_ref (log2 domain) ----
+        const float m_off = m_ref == -INFINITY ? 0.f : m_ref;
+        float tmax = -INFINITY;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                float x = HAS_BIAS ? fmaf(s[kb][v], p.scale_log2, bias_v[kb][v]) : s[kb][v] * p.scale_log2;
-                if (tail || diag) {
-                    const int key = key0 + kb * 32 + g * 16 + v;
-                    if (key >= p.Tk || (p.causal && key > q_row)) x = -INFINITY;
-                }
-                s[kb][v] = x;
-                mt = fmaxf(mt, x);
+                if constexpr (HAS_BIAS)
+                    s[kb][v] = fmaf(s[kb][v], p.scale_log2, fmaf(bias_v[kb][v], kLog2e, -m_off));
+                else
+                    s[kb][v] = fmaf(s[kb][v], p.scale_log2, -m_off);
             }
-        mt = fmaxf(mt, lane_xor32(mt));
-        const float m_new = fmaxf(m_run, mt);
-        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_safe);
-        m_run = m_new;
+        const bool diag = p.causal && (key0 + ATTN_BN - 1 > qb * ATTN_BM + wave * 32);
+        if (tail || diag) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int key = key0 + kb * 32 + g * 16 + v;
+                    if (key >= p.Tk || (p.causal && key > q_row)) s[kb][v] = -INFINITY;
+                }
+        }
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int v = 0; v < 16; v += 2) tmax = fmaxf(fmaxf(tmax, s[kb][v]), s[kb][v + 1]);
+        tmax = fmaxf(tmax, lane_xor32(tmax));
 
-        float lsum = 0.f;
+        // move the reference exponent only when needed (first finite logit of the row, or growth > 2^8)
+        const bool move = (m_ref == -INFINITY) ? (tmax != -INFINITY) : (tmax > ATTN_RESCALE_THRESHOLD);
+        if (__builtin_amdgcn_ballot_w64(move) != 0) {
+            const float shift = move ? tmax : 0.f;
+            const float alpha = move ? __builtin_amdgcn_exp2f(m_ref - (m_off + shift)) : 1.f;  // 0 when m_ref was -inf
+            m_ref = move ? m_off + shift : m_ref;
+            l_run *= alpha;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) s[kb][v] -= shift;
+#pragma unroll
+            for (int d = 0; d < NDB; ++d)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) oacc[d][v] *= alpha;
+        }
+
+        // ---- p = exp2(t), packed to the operand type ----
         uint32_t pk[2][8];
+        float lsum0 = 0.f, lsum1 = 0.f;  // the row sum uses the unrounded fp32 values: LSE keeps fp32 accuracy
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
             for (int v = 0; v < 16; v += 2) {
-                const float p0 = __builtin_amdgcn_exp2f(s[kb][v] - m_safe);
-                const float p1 = __builtin_amdgcn_exp2f(s[kb][v + 1] - m_safe);
-                lsum += p0 + p1;
+                const float p0 = __builtin_amdgcn_exp2f(s[kb][v]);
+                const float p1 = __builtin_amdgcn_exp2f(s[kb][v + 1]);
                 pk[kb][v / 2] = pack2<T>(p0, p1);
+                lsum0 += p0;
+                lsum1 += p1;
             }
-        l_run = l_run * alpha + lsum;
-#pragma unroll
-        for (int d = 0; d < NDB; ++d)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) oacc[d][v] *= alpha;
+        l_run += lsum0 + lsum1;
 
         // ---- O^T += V^T . P^T ----
-        const T* vt = vt_base + buf * SM::V_ELEMS;
+        const T* vs = vs_base + buf * TILE + tr_off;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             const int kb = t >> 1, jj = t & 1;
@@ -224,8 +250,10 @@ __global__ __launch_bounds__(ATTN_THREADS) void attn_fwd_kernel(const AttnFwdPar
             const typename MM::V8 pb = as_v8<T>(praw);
 #pragma unroll
             for (int d = 0; d < NDB; ++d) {
-                const u32x4 a =
-                    *reinterpret_cast<const u32x4*>(vt + (d * 32 + krow) * SM::VS + kb * 32 + g * 16 + jj * 8);
+                const T* src = vs + (kb * 32 + jj * 8) * ST + d * 32;
+                const u32x2 lo = lds_read_tr<T>(src);
+                const u32x2 hi = lds_read_tr<T>(src + 4 * ST);
+                const u32x4 a = {lo[0], lo[1], hi[0], hi[1]};
                 oacc[d] = MM::run(as_v8<T>(a), pb, oacc[d]);
             }
         }
@@ -262,7 +290,7 @@ __global__ __launch_bounds__(ATTN_THREADS) void attn_fwd_kernel(const AttnFwdPar
     }
     if (g == 0 && q_row < p.Tq_rounded) {
         // natural-log logsumexp; padding rows get a fixed value
-        const float lse = q_valid ? (m_run + __builtin_amdgcn_logf(l_tot)) * kLn2 : 0.f;
+        const float lse = q_valid ? (m_ref + __builtin_amdgcn_logf(l_tot)) * kLn2 : 0.f;
         p.lse[(int64_t)bh * p.Tq_rounded + q_row] = lse;
     }
 }

@@ -106,7 +106,11 @@ __device__ __forceinline__ void store_chunk(T* __restrict__ p, int first, int li
                 for (int e = 0; e < EPV; ++e) tmp[e] = from_f32<T>(in[v * EPV + e]);
                 u32x4 raw;
                 __builtin_memcpy(&raw, tmp, 16);
+#if defined(RGD_NT_STORE)
+                __builtin_nontemporal_store(raw, vp + v);
+#else
                 vp[v] = raw;
+#endif
             }
         }
     } else {
@@ -131,7 +135,13 @@ template <typename T, int N, bool VECTOR> struct Chunk {
         if constexpr (VEC) {
             const u32x4* p = reinterpret_cast<const u32x4*>(row + (first < limit ? first : 0));
 #pragma unroll
-            for (int i = 0; i < NVEC; ++i) v[i] = p[i];
+            for (int i = 0; i < NVEC; ++i) {
+#if defined(RGD_NT_LOAD)
+                v[i] = __builtin_nontemporal_load(p + i);
+#else
+                v[i] = p[i];
+#endif
+            }
         } else {
 #pragma unroll
             for (int e = 0; e < N; ++e) s[e] = row[first + e < limit ? first + e : 0];

@@ -187,7 +187,13 @@ struct HeadConfig {
     bool vector;
     bool table_f32;  // rotary table is fp32 while the tensors are 16-bit
 };
+#ifndef RGD_HEAD_U_FWD
+#define RGD_HEAD_U_FWD 4
+#endif
+#ifndef RGD_HEAD_U_BWD
+#define RGD_HEAD_U_BWD 2
+#endif
 constexpr int head_unroll(int mode, int nv) {
-    return nv > 1 ? 1 : ((mode == HEAD_LN_BWD || mode == HEAD_LNROPE_BWD) ? 2 : 4);
+    return nv > 1 ? 1 : ((mode == HEAD_LN_BWD || mode == HEAD_LNROPE_BWD) ? RGD_HEAD_U_BWD : RGD_HEAD_U_FWD);
 }
 template <typename T> int head_dispatch(const HeadConfig& cfg, const HeadParams& p, dim3 grid, hipStream_t s);
