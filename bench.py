@@ -59,18 +59,29 @@ def timed_loop(torch, step_fns, steps, warmup):
     n = len(step_fns)
     for i in range(warmup):
         step_fns[i % n](None)
+    # timed region: exactly `steps` steps between two synchronisations; only the two bracketing events
+    # are on the stream, so the launches run back to back
     torch.cuda.synchronize()
-    evs = []
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
+    e0.record()
     for i in range(steps):
-        rec = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
-        step_fns[i % n](rec)
-        evs.append(rec)
+        step_fns[i % n](None)
+    e1.record()
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) * 1e3 / steps
+    gpu_span = e0.elapsed_time(e1) / steps
+    # the same steps again with an event after every launch: per-kernel durations for the roofline
+    # (an event between two launches costs a few microseconds of stream time, which is why this is a
+    # separate pass and not the one `value` comes from)
+    evs = []
+    for i in range(steps):
+        rec = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+        step_fns[(i + steps) % n](rec)
+        evs.append(rec)
+    torch.cuda.synchronize()
     fwd = [e[0].elapsed_time(e[1]) for e in evs]
     bwd = [e[1].elapsed_time(e[2]) for e in evs]
-    gpu_span = evs[0][0].elapsed_time(evs[-1][2]) / steps
     return wall, gpu_span, fwd, bwd
 
 

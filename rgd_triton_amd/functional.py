@@ -299,7 +299,16 @@ def _cutoffs(seq_cutoff, tq, tk):
     return int(seq_cutoff), int(seq_cutoff)
 
 
+def _table_for(pos_emb, x):
+    """A rotary table the kernels can read next to tensors of x.dtype: same dtype, or fp32."""
+    if pos_emb.dtype == x.dtype or pos_emb.dtype == torch.float32:
+        return pos_emb
+    return pos_emb.float()  # e.g. an fp16 table with bf16 tensors: exact upcast, tiny tensor
+
+
 def _pos_emb_args(pos_emb, tq, tk):
+    """pos_emb (2, P, R) -> C arguments.  The kernels read a table in the tensors' dtype or in fp32; the
+    caller has already converted any other combination (see _table_for)."""
     assert pos_emb.ndim == 3 and pos_emb.shape[0] == 2, f"{pos_emb.shape=}"
     assert pos_emb.is_cuda and pos_emb.dtype in _FLOATS
     _, P, R = pos_emb.shape
@@ -351,7 +360,7 @@ class CombinedRoPEFunc(torch.autograd.Function):
     def forward(ctx, q, k, pos_emb, seq_cutoff=None, heads_second=True, in_place=False, kernel_cache=None):
         if in_place:
             assert q.stride(-1) == 1 and k.stride(-1) == 1, "in_place RoPE needs unit-stride head dims"
-        q, k, pos_emb = _lastdim_contig(q, k, pos_emb)
+        q, k, pos_emb = _lastdim_contig(q, k, _table_for(pos_emb, q))
         _seen(kernel_cache, "fwd", _sig(q, k, pos_emb) + (heads_second,))
         B, H, Tq, Tk, D = _qk_dims(q, k, heads_second, 128, "RoPE")
         pe = _pos_emb_args(pos_emb, Tq, Tk)
@@ -400,7 +409,7 @@ def triton_rope_fn(query, key, pos_emb, seq_cutoff=None, heads_second=True, fuse
 class FusedRoPEFunc(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, pos_emb, seq_cutoff=None, heads_second=True, norm_eps=1e-6, kernel_cache=None):
-        q, k, pos_emb = _lastdim_contig(q, k, pos_emb)
+        q, k, pos_emb = _lastdim_contig(q, k, _table_for(pos_emb, q))
         _seen(kernel_cache, "fwd", _sig(q, k, pos_emb) + (heads_second,))
         B, H, Tq, Tk, D = _qk_dims(q, k, heads_second, 128, "LayerNorm+RoPE")
         pe = _pos_emb_args(pos_emb, Tq, Tk)
