@@ -1,13 +1,13 @@
 // Attention backward as two deterministic kernels (no atomics, every gradient element written once):
 //
-//   attn_bwd_dq_kernel    one workgroup = 128 query rows; walks the keys.  Also produces
+//   attn_bwd_dq_kernel    one workgroup = 128 query rows; walks the keys in tiles of 64.  Also produces
 //                         delta = rowsum(O * dO) for the second kernel.
 //       S^T  = K . Q^T              A = K tile (LDS, row-major)       B = Q  (registers)
 //       dP^T = V . dO^T             A = V tile (LDS, row-major)       B = dO (registers)
-//       dS^T = P^T * (dP^T - delta) * scale,   P^T = exp2(S^T*c + bias*log2e - lse*log2e)
+//       dS^T = P^T * (dP^T - delta),   P^T = exp2(S^T*c + bias*log2e - lse*log2e)
 //       dQ^T += K^T . dS^T          A = K^T via transposing LDS reads  B = dS^T (registers)
 //
-//   attn_bwd_dkv_kernel   one workgroup = 128 keys; walks the query rows.
+//   attn_bwd_dkv_kernel   one workgroup = 128 keys; walks the query rows in tiles of 32.
 //       S  = Q . K^T                A = Q tile  (LDS, row-major)      B = K (registers)
 //       dP = dO . V^T               A = dO tile (LDS, row-major)      B = V (registers)
 //       dV^T += dO^T . P            A = dO^T via transposing reads    B = P  (registers)
@@ -15,9 +15,8 @@
 //
 // In both kernels the row/column that owns the output (query row for dQ, key for dK/dV) sits in one
 // lane column (lane % 32), so P and dS go from accumulator registers straight into the next matrix
-// product, and all LDS tiles are stored row-major exactly as they arrive from HBM.  Transposed
-// operands are fetched with ds_read_b64_tr_b16: inside each group of 16 lanes, result lane i gets
-// element (i % 4) of the 8-byte pieces addressed by lanes i/4, 4 + i/4, 8 + i/4 and 12 + i/4.
+// product, and all LDS tiles are stored row-major exactly as they arrive from HBM.  The softmax scale
+// is applied once to the finished dQ / dK accumulators instead of to every dS element.
 #pragma once
 
 #include "attn_common.h"
@@ -38,6 +37,27 @@ template <int DPAD> struct BwdTile {
     static constexpr int S = DPAD + 8;  // row stride of every staged tile (elements)
 };
 
+// writes 16 contiguous columns (two 16-byte stores on the vector path) of one output row
+template <typename T>
+__device__ __forceinline__ void store_row16(T* row, int col, int D, bool vec, const f32x16& acc, float mul) {
+    if (vec) {
+        if (col < D) {
+            Pack16 lo, hi;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                lo.w[e] = pack2<T>(acc[2 * e] * mul, acc[2 * e + 1] * mul);
+                hi.w[e] = pack2<T>(acc[8 + 2 * e] * mul, acc[8 + 2 * e + 1] * mul);
+            }
+            *reinterpret_cast<u32x4*>(row + col) = lo.v;
+            if (col + 8 < D) *reinterpret_cast<u32x4*>(row + col + 8) = hi.v;
+        }
+    } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+            if (col + v < D) row[col + v] = static_cast<T>(acc[v] * mul);
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 // dQ kernel
 // ------------------------------------------------------------------------------------------------
@@ -48,7 +68,7 @@ template <int DPAD> struct DqSmem {
 };
 
 template <typename T, int DPAD, bool HAS_BIAS>
-__global__ __launch_bounds__(BWD_THREADS) void attn_bwd_dq_kernel(const AttnBwdParams p) {
+__global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dq_kernel(const AttnBwdParams p) {
     typedef Mfma<T> MM;
     constexpr int BN = DqSmem<DPAD>::BN;
     constexpr int ST = BwdTile<DPAD>::S;
@@ -56,7 +76,9 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_dq_kernel(const AttnBwdP
     constexpr int NC = DPAD / 16;
     constexpr int NDB = DPAD / 32;
     constexpr int CPR = DPAD / 8;
-    constexpr int LOADS = BN * CPR / BWD_THREADS;
+    constexpr int TASKS = BN * CPR;
+    static_assert(TASKS % BWD_THREADS == 0, "tile chunks must divide evenly over the workgroup");
+    constexpr int LOADS = TASKS / BWD_THREADS;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     T* const ks_base = reinterpret_cast<T*>(smem_raw);
@@ -74,8 +96,6 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_dq_kernel(const AttnBwdP
     const T* qp = static_cast<const T*>(p.q.ptr) + b * p.q.sb + h * p.q.sh + (int64_t)q_ld * p.q.sn;
     const T* dop = static_cast<const T*>(p.dout.ptr) + b * p.dout.sb + h * p.dout.sh + (int64_t)q_ld * p.dout.sn;
     const T* op = static_cast<const T*>(p.o.ptr) + b * p.o.sb + h * p.o.sh + (int64_t)q_ld * p.o.sn;
-    const T* kp = static_cast<const T*>(p.k.ptr) + b * p.k.sb + h * p.k.sh;
-    const T* vp = static_cast<const T*>(p.v.ptr) + b * p.v.sb + h * p.v.sh;
 
     typename MM::V8 qreg[NC], doreg[NC];
     float dsum = 0.f;
@@ -92,7 +112,7 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_dq_kernel(const AttnBwdP
     const float delta = dsum + lane_xor32(dsum);
     const float lse = p.lse[(int64_t)bh * p.Tq_rounded + min(q_row, p.Tq_rounded - 1)];
     // rows that do not exist, and rows whose logits are all -inf, get probability 0 everywhere
-    const float lse_l2 = (q_valid && lse != -INFINITY) ? lse * kLog2e : INFINITY;
+    const float neg_lse_l2 = (q_valid && lse != -INFINITY) ? -lse * kLog2e : -INFINITY;
     if (g == 0 && q_row < p.Tq_rounded) p.delta[(int64_t)bh * p.Tq_rounded + q_row] = q_valid ? delta : 0.f;
 
     f32x16 acc[NDB];
@@ -104,25 +124,44 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_dq_kernel(const AttnBwdP
     int ntiles = (p.Tk + BN - 1) / BN;
     if (p.causal) ntiles = min(ntiles, (min(p.Tq, (qb + 1) * BWD_BM) + BN - 1) / BN);
 
+    const T* kbase = static_cast<const T*>(p.k.ptr) + b * p.k.sb + h * p.k.sh;
+    const T* vbase = static_cast<const T*>(p.v.ptr) + b * p.v.sb + h * p.v.sh;
+    int ld_key[LOADS], ld_dc[LOADS], koff[LOADS], voff[LOADS], soff[LOADS];
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+        const int id = tid + i * BWD_THREADS;
+        ld_key[i] = id / CPR;
+        ld_dc[i] = id % CPR;
+        koff[i] = ld_key[i] * (int)p.k.sn + ld_dc[i] * 8;
+        voff[i] = ld_key[i] * (int)p.v.sn + ld_dc[i] * 8;
+        soff[i] = ld_key[i] * ST + ld_dc[i] * 8;
+    }
+    const bool fast_tiles = vec && p.D == DPAD;
     u32x4 kst[LOADS], vst[LOADS];
     auto issue_loads = [&](int tile) {
         const int key0 = tile * BN;
+        const T* kt = kbase + (int64_t)key0 * p.k.sn;
+        const T* vt = vbase + (int64_t)key0 * p.v.sn;
+        if (fast_tiles && key0 + BN <= p.Tk) {
 #pragma unroll
-        for (int i = 0; i < LOADS; ++i) {
-            const int id = tid + i * BWD_THREADS;
-            const int key = id / CPR, dc = id % CPR;
-            const bool ok = key0 + key < p.Tk;
-            kst[i] = load8<T>(kp + (int64_t)(key0 + key) * p.k.sn, dc * 8, p.D, ok, vec);
-            vst[i] = load8<T>(vp + (int64_t)(key0 + key) * p.v.sn, dc * 8, p.D, ok, vec);
+            for (int i = 0; i < LOADS; ++i) {
+                kst[i] = *reinterpret_cast<const u32x4*>(kt + koff[i]);
+                vst[i] = *reinterpret_cast<const u32x4*>(vt + voff[i]);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < LOADS; ++i) {
+                const bool ok = key0 + ld_key[i] < p.Tk;
+                kst[i] = load8<T>(kt + (int64_t)ld_key[i] * p.k.sn, ld_dc[i] * 8, p.D, ok, vec);
+                vst[i] = load8<T>(vt + (int64_t)ld_key[i] * p.v.sn, ld_dc[i] * 8, p.D, ok, vec);
+            }
         }
     };
     auto store_tiles = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < LOADS; ++i) {
-            const int id = tid + i * BWD_THREADS;
-            const int key = id / CPR, dc = id % CPR;
-            *reinterpret_cast<u32x4*>(ks_base + buf * TILE + key * ST + dc * 8) = kst[i];
-            *reinterpret_cast<u32x4*>(vs_base + buf * TILE + key * ST + dc * 8) = vst[i];
+            *reinterpret_cast<u32x4*>(ks_base + buf * TILE + soff[i]) = kst[i];
+            *reinterpret_cast<u32x4*>(vs_base + buf * TILE + soff[i]) = vst[i];
         }
     };
     if (ntiles > 0) {
@@ -131,7 +170,8 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_dq_kernel(const AttnBwdP
     }
     __syncthreads();
 
-    const int krow = mfma_row_perm(li);
+    const int a_off = mfma_row_perm(li) * ST + g * 8;
+    const int tr_off = ((lane & 15) >> 2) * ST + mfma_row_perm(((lane >> 4) & 1) * 16 + (lane & 3) * 4) + g * 16 * ST;
     const char* bias_base = nullptr;
     int64_t bias_row = 0;
     if constexpr (HAS_BIAS) {
@@ -148,11 +188,11 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_dq_kernel(const AttnBwdP
         if constexpr (HAS_BIAS) {
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
-                load_bias16(bias_base, bias_row, p.bias_dtype, key0 + kb * 32 + g * 16, p.Tk, p.bias_vec && !tail, kLog2e,
+                load_bias16(bias_base, bias_row, p.bias_dtype, key0 + kb * 32 + g * 16, p.Tk, p.bias_vec && !tail, 1.0f,
                             bias_v[kb]);
         }
-        const T* ks = ks_base + buf * TILE;
-        const T* vs = vs_base + buf * TILE;
+        const T* ks = ks_base + buf * TILE + a_off;
+        const T* vs = vs_base + buf * TILE + a_off;
         f32x16 s[2], dp[2];
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
@@ -163,32 +203,43 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_dq_kernel(const AttnBwdP
             }
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
-                const u32x4 ka = *reinterpret_cast<const u32x4*>(ks + (kb * 32 + krow) * ST + c * 16 + g * 8);
+                const u32x4 ka = *reinterpret_cast<const u32x4*>(ks + kb * 32 * ST + c * 16);
                 s[kb] = MM::run(as_v8<T>(ka), qreg[c], s[kb]);
-                const u32x4 va = *reinterpret_cast<const u32x4*>(vs + (kb * 32 + krow) * ST + c * 16 + g * 8);
+                const u32x4 va = *reinterpret_cast<const u32x4*>(vs + kb * 32 * ST + c * 16);
                 dp[kb] = MM::run(as_v8<T>(va), doreg[c], dp[kb]);
             }
         }
+        // t = logit - lse (log2 domain)
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                if constexpr (HAS_BIAS)
+                    s[kb][v] = fmaf(s[kb][v], p.scale_log2, fmaf(bias_v[kb][v], kLog2e, neg_lse_l2));
+                else
+                    s[kb][v] = fmaf(s[kb][v], p.scale_log2, neg_lse_l2);
+            }
         const bool diag = p.causal && (key0 + BN - 1 > qb * BWD_BM + wave * 32);
+        if (tail || diag) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int key = key0 + kb * 32 + g * 16 + v;
+                    if (key >= p.Tk || (p.causal && key > q_row)) s[kb][v] = -INFINITY;
+                }
+        }
         uint32_t dsk[2][8];
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
             for (int v = 0; v < 16; v += 2) {
-                float dsv[2];
-#pragma unroll
-                for (int e = 0; e < 2; ++e) {
-                    float x = HAS_BIAS ? fmaf(s[kb][v + e], p.scale_log2, bias_v[kb][v + e]) : s[kb][v + e] * p.scale_log2;
-                    if (tail || diag) {
-                        const int key = key0 + kb * 32 + g * 16 + v + e;
-                        if (key >= p.Tk || (p.causal && key > q_row)) x = -INFINITY;
-                    }
-                    const float pr = __builtin_amdgcn_exp2f(x - lse_l2);
-                    dsv[e] = pr * (dp[kb][v + e] - delta) * p.scale;
-                }
-                dsk[kb][v / 2] = pack2<T>(dsv[0], dsv[1]);
+                const float p0 = __builtin_amdgcn_exp2f(s[kb][v]);
+                const float p1 = __builtin_amdgcn_exp2f(s[kb][v + 1]);
+                dsk[kb][v / 2] = pack2<T>(p0 * (dp[kb][v] - delta), p1 * (dp[kb][v + 1] - delta));
             }
         // dQ^T += K^T . dS^T
+        const T* kt = ks_base + buf * TILE + tr_off;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             const int kb = t >> 1, jj = t & 1;
@@ -196,8 +247,11 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_dq_kernel(const AttnBwdP
             const typename MM::V8 bop = as_v8<T>(raw);
 #pragma unroll
             for (int d = 0; d < NDB; ++d) {
-                const typename MM::V8 a = load_a_transposed<T>(ks, ST, kb * 32 + g * 16 + jj * 8, d * 32, lane);
-                acc[d] = MM::run(a, bop, acc[d]);
+                const T* src = kt + (kb * 32 + jj * 8) * ST + d * 32;
+                const u32x2 lo = lds_read_tr<T>(src);
+                const u32x2 hi = lds_read_tr<T>(src + 4 * ST);
+                const u32x4 a = {lo[0], lo[1], hi[0], hi[1]};
+                acc[d] = MM::run(as_v8<T>(a), bop, acc[d]);
             }
         }
         if (j + 1 < ntiles) store_tiles(buf ^ 1);
@@ -207,25 +261,7 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_dq_kernel(const AttnBwdP
     if (q_valid) {
         T* dqp = static_cast<T*>(const_cast<void*>(p.dq.ptr)) + b * p.dq.sb + h * p.dq.sh + (int64_t)q_row * p.dq.sn;
 #pragma unroll
-        for (int d = 0; d < NDB; ++d) {
-            const int col = d * 32 + g * 16;
-            if (vec) {
-                if (col < p.D) {
-                    Pack16 lo, hi;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        lo.w[e] = pack2<T>(acc[d][2 * e], acc[d][2 * e + 1]);
-                        hi.w[e] = pack2<T>(acc[d][8 + 2 * e], acc[d][8 + 2 * e + 1]);
-                    }
-                    *reinterpret_cast<u32x4*>(dqp + col) = lo.v;
-                    if (col + 8 < p.D) *reinterpret_cast<u32x4*>(dqp + col + 8) = hi.v;
-                }
-            } else {
-#pragma unroll
-                for (int v = 0; v < 16; ++v)
-                    if (col + v < p.D) dqp[col + v] = static_cast<T>(acc[d][v]);
-            }
-        }
+        for (int d = 0; d < NDB; ++d) store_row16<T>(dqp, d * 32 + g * 16, p.D, vec, acc[d], p.scale);
     }
 }
 
@@ -233,25 +269,42 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_dq_kernel(const AttnBwdP
 // dK / dV kernel
 // ------------------------------------------------------------------------------------------------
 template <int DPAD> struct DkvSmem {
-    static constexpr int BQ = DPAD <= 64 ? 64 : 32;  // query rows per tile
+    static constexpr int BQ = 32;  // query rows per tile
     static constexpr int TILE = BQ * BwdTile<DPAD>::S;
-    // per buffer: Q tile, dO tile, then BQ floats of lse*log2e and BQ floats of delta
+    // per buffer: Q tile, dO tile, then BQ floats of -lse*log2e and BQ floats of delta
     static constexpr int BUF_BYTES = 2 * TILE * 2 + 2 * BQ * 4;
     static constexpr size_t BYTES = 2 * BUF_BYTES;
 };
 
+// 16 bias values of one key column: rows q0 + 16g .. +15 of the bias matrix, element type TB.
+// `rows_ok` = all 16 rows exist; otherwise rows >= Tq read the last existing row (masked out later).
+template <typename TB>
+__device__ __forceinline__ void load_bias_column(const char* col_base, int64_t sn, int q_first, int Tq, bool rows_ok,
+                                                 float (&out)[16]) {
+    const TB* base = reinterpret_cast<const TB*>(col_base);
+    TB raw[16];
+    if (rows_ok) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) raw[v] = base[(int64_t)(q_first + v) * sn];
+    } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) raw[v] = base[(int64_t)min(q_first + v, Tq - 1) * sn];
+    }
+#pragma unroll
+    for (int v = 0; v < 16; ++v) out[v] = static_cast<float>(raw[v]);
+}
+
 template <typename T, int DPAD, bool HAS_BIAS>
-__global__ __launch_bounds__(BWD_THREADS) void attn_bwd_dkv_kernel(const AttnBwdParams p) {
+__global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dkv_kernel(const AttnBwdParams p) {
     typedef Mfma<T> MM;
     constexpr int BQ = DkvSmem<DPAD>::BQ;
-    constexpr int NQB = BQ / 32;
     constexpr int ST = BwdTile<DPAD>::S;
     constexpr int TILE = DkvSmem<DPAD>::TILE;
     constexpr int BUFB = DkvSmem<DPAD>::BUF_BYTES;
     constexpr int NC = DPAD / 16;
     constexpr int NDB = DPAD / 32;
     constexpr int CPR = DPAD / 8;
-    constexpr int TASKS = BQ * CPR;
+    constexpr int TASKS = BQ * CPR;  // 16-byte chunks of one tile: 128 .. 512
     constexpr int LOADS = (TASKS + BWD_THREADS - 1) / BWD_THREADS;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -267,8 +320,8 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_dkv_kernel(const AttnBwd
 
     const T* kp = static_cast<const T*>(p.k.ptr) + b * p.k.sb + h * p.k.sh + (int64_t)k_ld * p.k.sn;
     const T* vp = static_cast<const T*>(p.v.ptr) + b * p.v.sb + h * p.v.sh + (int64_t)k_ld * p.v.sn;
-    const T* qp = static_cast<const T*>(p.q.ptr) + b * p.q.sb + h * p.q.sh;
-    const T* dop = static_cast<const T*>(p.dout.ptr) + b * p.dout.sb + h * p.dout.sh;
+    const T* qbase = static_cast<const T*>(p.q.ptr) + b * p.q.sb + h * p.q.sh;
+    const T* dobase = static_cast<const T*>(p.dout.ptr) + b * p.dout.sb + h * p.dout.sh;
     const float* lsep = p.lse + (int64_t)bh * p.Tq_rounded;
     const float* deltap = p.delta + (int64_t)bh * p.Tq_rounded;
 
@@ -290,23 +343,46 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_dkv_kernel(const AttnBwd
     const int ntiles = (p.Tq + BQ - 1) / BQ;
     const int tile_begin = p.causal ? min(ntiles, (kblk * BWD_BM) / BQ) : 0;
 
+    int ld_row[LOADS], ld_dc[LOADS], qoff[LOADS], dooff[LOADS], soff[LOADS];
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+        const int id = tid + i * BWD_THREADS;
+        ld_row[i] = id / CPR;
+        ld_dc[i] = id % CPR;
+        qoff[i] = ld_row[i] * (int)p.q.sn + ld_dc[i] * 8;
+        dooff[i] = ld_row[i] * (int)p.dout.sn + ld_dc[i] * 8;
+        soff[i] = ld_row[i] * ST + ld_dc[i] * 8;
+    }
+    const bool fast_tiles = vec && p.D == DPAD;
     u32x4 qst[LOADS], dst[LOADS];
     float lse_st = 0.f, delta_st = 0.f;
     auto issue_loads = [&](int tile) {
         const int q0 = tile * BQ;
+        const T* qt = qbase + (int64_t)q0 * p.q.sn;
+        const T* dot = dobase + (int64_t)q0 * p.dout.sn;
+        if (fast_tiles && q0 + BQ <= p.Tq) {
 #pragma unroll
-        for (int i = 0; i < LOADS; ++i) {
-            const int id = tid + i * BWD_THREADS;
-            const int r = id / CPR, dc = id % CPR;
-            const bool ok = id < TASKS && q0 + r < p.Tq;
-            qst[i] = load8<T>(qp + (int64_t)(q0 + r) * p.q.sn, dc * 8, p.D, ok, vec);
-            dst[i] = load8<T>(dop + (int64_t)(q0 + r) * p.dout.sn, dc * 8, p.D, ok, vec);
+            for (int i = 0; i < LOADS; ++i) {
+                if (TASKS % BWD_THREADS == 0 || tid + i * BWD_THREADS < TASKS) {
+                    qst[i] = *reinterpret_cast<const u32x4*>(qt + qoff[i]);
+                    dst[i] = *reinterpret_cast<const u32x4*>(dot + dooff[i]);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < LOADS; ++i) {
+                const bool ok = tid + i * BWD_THREADS < TASKS && q0 + ld_row[i] < p.Tq;
+                qst[i] = load8<T>(qt + (int64_t)ld_row[i] * p.q.sn, ld_dc[i] * 8, p.D, ok, vec);
+                dst[i] = load8<T>(dot + (int64_t)ld_row[i] * p.dout.sn, ld_dc[i] * 8, p.D, ok, vec);
+            }
         }
         if (tid < BQ) {
             const int q = q0 + tid;
-            const float l = q < p.Tq ? lsep[q] : 0.f;
-            lse_st = (q < p.Tq && l != -INFINITY) ? l * kLog2e : INFINITY;
-            delta_st = q < p.Tq ? deltap[q] : 0.f;
+            const bool ok = q < p.Tq;
+            const float l = lsep[ok ? q : 0];
+            // rows that do not exist or have no finite logit get probability 0 (exp2(-inf))
+            lse_st = (ok && l != -INFINITY) ? -l * kLog2e : -INFINITY;
+            delta_st = ok ? deltap[q] : 0.f;
         }
     };
     auto store_tiles = [&](int buf) {
@@ -315,11 +391,9 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_dkv_kernel(const AttnBwd
         float* st = reinterpret_cast<float*>(smem_raw + buf * BUFB + 2 * TILE * 2);
 #pragma unroll
         for (int i = 0; i < LOADS; ++i) {
-            const int id = tid + i * BWD_THREADS;
-            const int r = id / CPR, dc = id % CPR;
-            if (id < TASKS) {
-                *reinterpret_cast<u32x4*>(qs + r * ST + dc * 8) = qst[i];
-                *reinterpret_cast<u32x4*>(ds + r * ST + dc * 8) = dst[i];
+            if (TASKS % BWD_THREADS == 0 || tid + i * BWD_THREADS < TASKS) {
+                *reinterpret_cast<u32x4*>(qs + soff[i]) = qst[i];
+                *reinterpret_cast<u32x4*>(ds + soff[i]) = dst[i];
             }
         }
         if (tid < BQ) {
@@ -333,15 +407,17 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_dkv_kernel(const AttnBwd
     }
     __syncthreads();
 
-    const int arow = mfma_row_perm(li);
+    const int a_off = mfma_row_perm(li) * ST + g * 8;
+    const int tr_off = ((lane & 15) >> 2) * ST + mfma_row_perm(((lane >> 4) & 1) * 16 + (lane & 3) * 4) + g * 16 * ST;
+
     const int besz = p.bias_dtype == RGD_F32 ? 4 : 2;
-    const char* bias_base = nullptr;
+    const char* bias_col = nullptr;  // this lane's key column of the bias, at row 16g
     float bias_vector = 0.f;
     if constexpr (HAS_BIAS) {
-        bias_base = static_cast<const char*>(p.bias.ptr) + (b * p.bias.sb + h * p.bias.sh + k_ld) * besz;
+        bias_col = static_cast<const char*>(p.bias.ptr) + (b * p.bias.sb + h * p.bias.sh + k_ld) * besz;
         if (p.bias_kind == RGD_BIAS_VECTOR) {
             float t[1];
-            load_chunk_dyn<1, false>(bias_base, p.bias_dtype, 0, 1, t);
+            load_chunk_dyn<1, false>(bias_col, p.bias_dtype, 0, 1, t);
             bias_vector = t[0] * kLog2e;
         }
     }
@@ -351,79 +427,91 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_dkv_kernel(const AttnBwd
         const int q0 = j * BQ;
         if (j + 1 < ntiles) issue_loads(j + 1);
 
+        float bias_r[16];
+        if constexpr (HAS_BIAS) {
+            if (p.bias_kind == RGD_BIAS_MATRIX) {
+                const bool rows_ok = q0 + BQ <= p.Tq;
+                const int qf = q0 + g * 16;
+                if (p.bias_dtype == RGD_BF16)
+                    load_bias_column<bf16_t>(bias_col, p.bias.sn, qf, p.Tq, rows_ok, bias_r);
+                else if (p.bias_dtype == RGD_F16)
+                    load_bias_column<f16_t>(bias_col, p.bias.sn, qf, p.Tq, rows_ok, bias_r);
+                else
+                    load_bias_column<float>(bias_col, p.bias.sn, qf, p.Tq, rows_ok, bias_r);
+            }
+        }
+
         const T* qs = reinterpret_cast<const T*>(smem_raw + buf * BUFB);
-        const T* ds_t = qs + TILE;
+        const T* dos = qs + TILE;
         const float* st = reinterpret_cast<const float*>(smem_raw + buf * BUFB + 2 * TILE * 2);
 
-        f32x16 s[NQB], dp[NQB];
+        f32x16 s, dp;
 #pragma unroll
-        for (int qb = 0; qb < NQB; ++qb) {
+        for (int v = 0; v < 16; ++v) {
+            s[v] = 0.f;
+            dp[v] = 0.f;
+        }
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                s[qb][v] = 0.f;
-                dp[qb][v] = 0.f;
+        for (int c = 0; c < NC; ++c) {
+            const u32x4 qa = *reinterpret_cast<const u32x4*>(qs + a_off + c * 16);
+            s = MM::run(as_v8<T>(qa), kreg[c], s);
+            const u32x4 da = *reinterpret_cast<const u32x4*>(dos + a_off + c * 16);
+            dp = MM::run(as_v8<T>(da), vreg[c], dp);
+        }
+        float nlse[16], dlt[16];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const f32x4 a = *reinterpret_cast<const f32x4*>(st + g * 16 + 4 * i);
+            const f32x4 c = *reinterpret_cast<const f32x4*>(st + BQ + g * 16 + 4 * i);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                nlse[4 * i + e] = a[e];
+                dlt[4 * i + e] = c[e];
             }
+        }
 #pragma unroll
-            for (int c = 0; c < NC; ++c) {
-                const u32x4 qa = *reinterpret_cast<const u32x4*>(qs + (qb * 32 + arow) * ST + c * 16 + g * 8);
-                s[qb] = MM::run(as_v8<T>(qa), kreg[c], s[qb]);
-                const u32x4 da = *reinterpret_cast<const u32x4*>(ds_t + (qb * 32 + arow) * ST + c * 16 + g * 8);
-                dp[qb] = MM::run(as_v8<T>(da), vreg[c], dp[qb]);
+        for (int v = 0; v < 16; ++v) {
+            if constexpr (HAS_BIAS) {
+                const float bl = p.bias_kind == RGD_BIAS_VECTOR ? bias_vector + nlse[v] : fmaf(bias_r[v], kLog2e, nlse[v]);
+                s[v] = fmaf(s[v], p.scale_log2, bl);
+            } else {
+                s[v] = fmaf(s[v], p.scale_log2, nlse[v]);
             }
         }
         const bool diag = p.causal && (q0 < kblk * BWD_BM + wave * 32 + 32);
-        uint32_t pk[NQB][8], dsk[NQB][8];
+        if (!k_valid || diag) {
 #pragma unroll
-        for (int qb = 0; qb < NQB; ++qb) {
-            float lse_r[16], delta_r[16];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const f32x4 a = *reinterpret_cast<const f32x4*>(st + qb * 32 + g * 16 + 4 * i);
-                const f32x4 c = *reinterpret_cast<const f32x4*>(st + BQ + qb * 32 + g * 16 + 4 * i);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    lse_r[4 * i + e] = a[e];
-                    delta_r[4 * i + e] = c[e];
-                }
+            for (int v = 0; v < 16; ++v) {
+                const int q = q0 + g * 16 + v;
+                if (!k_valid || key > q) s[v] = -INFINITY;
             }
+        }
+        uint32_t pk[8], dsk[8];
 #pragma unroll
-            for (int v = 0; v < 16; v += 2) {
-                float pv[2], dsv[2];
-#pragma unroll
-                for (int e = 0; e < 2; ++e) {
-                    const int q = q0 + qb * 32 + g * 16 + v + e;
-                    float x = s[qb][v + e] * p.scale_log2;
-                    if constexpr (HAS_BIAS) {
-                        if (p.bias_kind == RGD_BIAS_VECTOR) {
-                            x += bias_vector;
-                        } else {
-                            float t[1] = {0.f};
-                            if (q < p.Tq) load_chunk_dyn<1, false>(bias_base + (int64_t)q * p.bias.sn * besz, p.bias_dtype, 0, 1, t);
-                            x = fmaf(t[0], kLog2e, x);
-                        }
-                    }
-                    if (!k_valid || (diag && key > q)) x = -INFINITY;
-                    pv[e] = __builtin_amdgcn_exp2f(x - lse_r[v + e]);
-                    dsv[e] = pv[e] * (dp[qb][v + e] - delta_r[v + e]) * p.scale;
-                }
-                pk[qb][v / 2] = pack2<T>(pv[0], pv[1]);
-                dsk[qb][v / 2] = pack2<T>(dsv[0], dsv[1]);
-            }
+        for (int v = 0; v < 16; v += 2) {
+            const float p0 = __builtin_amdgcn_exp2f(s[v]);
+            const float p1 = __builtin_amdgcn_exp2f(s[v + 1]);
+            pk[v / 2] = pack2<T>(p0, p1);
+            dsk[v / 2] = pack2<T>(p0 * (dp[v] - dlt[v]), p1 * (dp[v + 1] - dlt[v + 1]));
         }
         // dV^T += dO^T . P ;  dK^T += Q^T . dS
 #pragma unroll
-        for (int t = 0; t < 2 * NQB; ++t) {
-            const int qb = t >> 1, jj = t & 1;
-            const u32x4 praw = {pk[qb][jj * 4 + 0], pk[qb][jj * 4 + 1], pk[qb][jj * 4 + 2], pk[qb][jj * 4 + 3]};
-            const u32x4 draw = {dsk[qb][jj * 4 + 0], dsk[qb][jj * 4 + 1], dsk[qb][jj * 4 + 2], dsk[qb][jj * 4 + 3]};
+        for (int jj = 0; jj < 2; ++jj) {
+            const u32x4 praw = {pk[jj * 4 + 0], pk[jj * 4 + 1], pk[jj * 4 + 2], pk[jj * 4 + 3]};
+            const u32x4 draw = {dsk[jj * 4 + 0], dsk[jj * 4 + 1], dsk[jj * 4 + 2], dsk[jj * 4 + 3]};
             const typename MM::V8 pb = as_v8<T>(praw), db = as_v8<T>(draw);
-            const int row0 = qb * 32 + g * 16 + jj * 8;
 #pragma unroll
             for (int d = 0; d < NDB; ++d) {
-                const typename MM::V8 at = load_a_transposed<T>(ds_t, ST, row0, d * 32, lane);
-                dv_acc[d] = MM::run(at, pb, dv_acc[d]);
-                const typename MM::V8 qt = load_a_transposed<T>(qs, ST, row0, d * 32, lane);
-                dk_acc[d] = MM::run(qt, db, dk_acc[d]);
+                const T* dsrc = dos + tr_off + jj * 8 * ST + d * 32;
+                const u32x2 dlo = lds_read_tr<T>(dsrc);
+                const u32x2 dhi = lds_read_tr<T>(dsrc + 4 * ST);
+                const u32x4 da = {dlo[0], dlo[1], dhi[0], dhi[1]};
+                dv_acc[d] = MM::run(as_v8<T>(da), pb, dv_acc[d]);
+                const T* qsrc = qs + tr_off + jj * 8 * ST + d * 32;
+                const u32x2 qlo = lds_read_tr<T>(qsrc);
+                const u32x2 qhi = lds_read_tr<T>(qsrc + 4 * ST);
+                const u32x4 qa = {qlo[0], qlo[1], qhi[0], qhi[1]};
+                dk_acc[d] = MM::run(as_v8<T>(qa), db, dk_acc[d]);
             }
         }
         if (j + 1 < ntiles) store_tiles(buf ^ 1);
@@ -435,32 +523,8 @@ __global__ __launch_bounds__(BWD_THREADS) void attn_bwd_dkv_kernel(const AttnBwd
         T* dvp = static_cast<T*>(const_cast<void*>(p.dv.ptr)) + b * p.dv.sb + h * p.dv.sh + (int64_t)key * p.dv.sn;
 #pragma unroll
         for (int d = 0; d < NDB; ++d) {
-            const int col = d * 32 + g * 16;
-            if (vec) {
-                if (col < p.D) {
-                    Pack16 a, c, e2, f;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        a.w[e] = pack2<T>(dk_acc[d][2 * e], dk_acc[d][2 * e + 1]);
-                        c.w[e] = pack2<T>(dk_acc[d][8 + 2 * e], dk_acc[d][8 + 2 * e + 1]);
-                        e2.w[e] = pack2<T>(dv_acc[d][2 * e], dv_acc[d][2 * e + 1]);
-                        f.w[e] = pack2<T>(dv_acc[d][8 + 2 * e], dv_acc[d][8 + 2 * e + 1]);
-                    }
-                    *reinterpret_cast<u32x4*>(dkp + col) = a.v;
-                    *reinterpret_cast<u32x4*>(dvp + col) = e2.v;
-                    if (col + 8 < p.D) {
-                        *reinterpret_cast<u32x4*>(dkp + col + 8) = c.v;
-                        *reinterpret_cast<u32x4*>(dvp + col + 8) = f.v;
-                    }
-                }
-            } else {
-#pragma unroll
-                for (int v = 0; v < 16; ++v)
-                    if (col + v < p.D) {
-                        dkp[col + v] = static_cast<T>(dk_acc[d][v]);
-                        dvp[col + v] = static_cast<T>(dv_acc[d][v]);
-                    }
-            }
+            store_row16<T>(dkp, d * 32 + g * 16, p.D, vec, dk_acc[d], p.scale);
+            store_row16<T>(dvp, d * 32 + g * 16, p.D, vec, dv_acc[d], 1.0f);
         }
     }
 }
