@@ -6,6 +6,10 @@
 #include <stdlib.h>
 #include <string.h>
 
+// kernel instantiations live in attn_f16.hip / attn_bf16.hip (attn_inst.h) so they compile in parallel
+template <typename T> int dispatch_fwd(const AttnFwdParams& p, unsigned grid, hipStream_t s);
+template <typename T, bool DQ> int dispatch_bwd(const AttnBwdParams& p, unsigned grid, hipStream_t s);
+
 namespace {
 
 bool t4_vec_ok(const rgd_tensor4* t) {
@@ -18,62 +22,6 @@ AttnTensor at(const rgd_tensor4* t) {
     a.sh = t ? t->stride_h : 0;
     a.sn = t ? t->stride_n : 0;
     return a;
-}
-
-template <typename T, int DPAD, bool HAS_BIAS> int launch_fwd(const AttnFwdParams& p, unsigned grid, hipStream_t s) {
-    auto kern = attn_fwd_kernel<T, DPAD, HAS_BIAS>;
-    constexpr size_t lds = AttnFwdSmem<DPAD>::BYTES;
-    static bool configured = false;  // benign race: the attribute is idempotent
-    if (!configured && lds > 48 * 1024) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)lds) != hipSuccess) {
-            rgd_set_error("rgd_attn_fwd: cannot reserve %zu bytes of LDS", lds);
-            return RGD_ERR_LAUNCH;
-        }
-        configured = true;
-    }
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(ATTN_THREADS), lds, s, p);
-    return RGD_OK;
-}
-
-template <typename T> int dispatch_fwd(const AttnFwdParams& p, unsigned grid, hipStream_t s) {
-    const bool hb = p.bias_kind != RGD_BIAS_NONE;
-#define FWD_CASE(DP)                                                             \
-    if (p.D <= DP) return hb ? launch_fwd<T, DP, true>(p, grid, s) : launch_fwd<T, DP, false>(p, grid, s);
-    FWD_CASE(32)
-    FWD_CASE(64)
-    FWD_CASE(96)
-    FWD_CASE(128)
-#undef FWD_CASE
-    return RGD_ERR_UNSUPPORTED;
-}
-
-template <typename T, int DPAD, bool HAS_BIAS, bool DQ> int launch_bwd(const AttnBwdParams& p, unsigned grid, hipStream_t s) {
-    auto kern = DQ ? attn_bwd_dq_kernel<T, DPAD, HAS_BIAS> : attn_bwd_dkv_kernel<T, DPAD, HAS_BIAS>;
-    constexpr size_t lds = DQ ? DqSmem<DPAD>::BYTES : DkvSmem<DPAD>::BYTES;
-    static bool configured = false;
-    if (!configured && lds > 48 * 1024) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)lds) != hipSuccess) {
-            rgd_set_error("rgd_attn_bwd: cannot reserve %zu bytes of LDS", lds);
-            return RGD_ERR_LAUNCH;
-        }
-        configured = true;
-    }
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(BWD_THREADS), lds, s, p);
-    return RGD_OK;
-}
-
-template <typename T, bool DQ> int dispatch_bwd(const AttnBwdParams& p, unsigned grid, hipStream_t s) {
-    const bool hb = p.bias_kind != RGD_BIAS_NONE;
-#define BWD_CASE(DP)                                                                     \
-    if (p.D <= DP) return hb ? launch_bwd<T, DP, true, DQ>(p, grid, s) : launch_bwd<T, DP, false, DQ>(p, grid, s);
-    BWD_CASE(32)
-    BWD_CASE(64)
-    BWD_CASE(96)
-    BWD_CASE(128)
-#undef BWD_CASE
-    return RGD_ERR_UNSUPPORTED;
 }
 
 int check_common(const char* name, int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, int dtype, int bias_kind,

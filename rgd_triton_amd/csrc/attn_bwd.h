@@ -67,8 +67,10 @@ template <int DPAD> struct DqSmem {
     static constexpr size_t BYTES = 2 * 2 * TILE * 2;  // K and V, double buffered
 };
 
-template <typename T, int DPAD, bool HAS_BIAS>
+template <typename T, int DPAD, int BIAS>
 __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dq_kernel(const AttnBwdParams p) {
+    constexpr bool HAS_BIAS = BIAS != BIAS_OFF;
+    typedef typename BiasElem<T, BIAS>::type TB;
     typedef Mfma<T> MM;
     constexpr int BN = DqSmem<DPAD>::BN;
     constexpr int ST = BwdTile<DPAD>::S;
@@ -172,25 +174,23 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dq_k
 
     const int a_off = mfma_row_perm(li) * ST + g * 8;
     const int tr_off = ((lane & 15) >> 2) * ST + mfma_row_perm(((lane >> 4) & 1) * 16 + (lane & 3) * 4) + g * 16 * ST;
-    const char* bias_base = nullptr;
-    int64_t bias_row = 0;
+    const TB* bias_row = nullptr;
+    BiasRuns<TB> bias_cur, bias_nxt;  // fetched one tile ahead of use
     if constexpr (HAS_BIAS) {
-        bias_base = static_cast<const char*>(p.bias.ptr);
-        bias_row = b * p.bias.sb + h * p.bias.sh + (int64_t)q_ld * p.bias.sn;
+        bias_row = static_cast<const TB*>(p.bias.ptr) + b * p.bias.sb + h * p.bias.sh + (int64_t)q_ld * p.bias.sn;
+        if (ntiles > 0) bias_cur.load(bias_row, 0, g, p.Tk, p.bias_vec && BN <= p.Tk);
     }
 
     for (int j = 0; j < ntiles; ++j) {
         const int buf = j & 1;
         const int key0 = j * BN;
-        if (j + 1 < ntiles) issue_loads(j + 1);
         const bool tail = key0 + BN > p.Tk;
-        float bias_v[2][16];
-        if constexpr (HAS_BIAS) {
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-                load_bias16(bias_base, bias_row, p.bias_dtype, key0 + kb * 32 + g * 16, p.Tk, p.bias_vec && !tail, 1.0f,
-                            bias_v[kb]);
+        if (j + 1 < ntiles) {
+            issue_loads(j + 1);
+            if constexpr (HAS_BIAS) bias_nxt.load(bias_row, key0 + BN, g, p.Tk, p.bias_vec && key0 + 2 * BN <= p.Tk);
         }
+        float bias_v[2][16];
+        if constexpr (HAS_BIAS) bias_cur.decode(bias_v);
         const T* ks = ks_base + buf * TILE + a_off;
         const T* vs = vs_base + buf * TILE + a_off;
         f32x16 s[2], dp[2];
@@ -254,7 +254,10 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dq_k
                 acc[d] = MM::run(as_v8<T>(a), bop, acc[d]);
             }
         }
-        if (j + 1 < ntiles) store_tiles(buf ^ 1);
+        if (j + 1 < ntiles) {
+            store_tiles(buf ^ 1);
+            if constexpr (HAS_BIAS) bias_cur = bias_nxt;
+        }
         __syncthreads();
     }
 
@@ -276,26 +279,30 @@ template <int DPAD> struct DkvSmem {
     static constexpr size_t BYTES = 2 * BUF_BYTES;
 };
 
-// 16 bias values of one key column: rows q0 + 16g .. +15 of the bias matrix, element type TB.
+// 16 bias values of one key column (rows q_first .. +15 of the bias matrix) in the "key per lane"
+// layout.  load() only issues the reads so it can run a tile ahead of decode().
 // `rows_ok` = all 16 rows exist; otherwise rows >= Tq read the last existing row (masked out later).
-template <typename TB>
-__device__ __forceinline__ void load_bias_column(const char* col_base, int64_t sn, int q_first, int Tq, bool rows_ok,
-                                                 float (&out)[16]) {
-    const TB* base = reinterpret_cast<const TB*>(col_base);
+template <typename TB> struct BiasColumn {
     TB raw[16];
-    if (rows_ok) {
+    __device__ __forceinline__ void load(const TB* __restrict__ col, int64_t sn, int q_first, int Tq, bool rows_ok) {
+        if (rows_ok) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) raw[v] = base[(int64_t)(q_first + v) * sn];
-    } else {
+            for (int v = 0; v < 16; ++v) raw[v] = col[(int64_t)(q_first + v) * sn];
+        } else {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) raw[v] = base[(int64_t)min(q_first + v, Tq - 1) * sn];
+            for (int v = 0; v < 16; ++v) raw[v] = col[(int64_t)min(q_first + v, Tq - 1) * sn];
+        }
     }
+    __device__ __forceinline__ void decode(float (&out)[16]) const {
 #pragma unroll
-    for (int v = 0; v < 16; ++v) out[v] = static_cast<float>(raw[v]);
-}
+        for (int v = 0; v < 16; ++v) out[v] = static_cast<float>(raw[v]);
+    }
+};
 
-template <typename T, int DPAD, bool HAS_BIAS>
+template <typename T, int DPAD, int BIAS>
 __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dkv_kernel(const AttnBwdParams p) {
+    constexpr bool HAS_BIAS = BIAS != BIAS_OFF;
+    typedef typename BiasElem<T, BIAS>::type TB;
     typedef Mfma<T> MM;
     constexpr int BQ = DkvSmem<DPAD>::BQ;
     constexpr int ST = BwdTile<DPAD>::S;
@@ -410,35 +417,30 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dkv_
     const int a_off = mfma_row_perm(li) * ST + g * 8;
     const int tr_off = ((lane & 15) >> 2) * ST + mfma_row_perm(((lane >> 4) & 1) * 16 + (lane & 3) * 4) + g * 16 * ST;
 
-    const int besz = p.bias_dtype == RGD_F32 ? 4 : 2;
-    const char* bias_col = nullptr;  // this lane's key column of the bias, at row 16g
+    const TB* bias_col = nullptr;  // this lane's key column of the bias
     float bias_vector = 0.f;
+    const bool bias_matrix = HAS_BIAS && p.bias_kind == RGD_BIAS_MATRIX;
+    BiasColumn<TB> bias_cur, bias_nxt;  // fetched one tile ahead of use
     if constexpr (HAS_BIAS) {
-        bias_col = static_cast<const char*>(p.bias.ptr) + (b * p.bias.sb + h * p.bias.sh + k_ld) * besz;
-        if (p.bias_kind == RGD_BIAS_VECTOR) {
-            float t[1];
-            load_chunk_dyn<1, false>(bias_col, p.bias_dtype, 0, 1, t);
-            bias_vector = t[0] * kLog2e;
-        }
+        bias_col = static_cast<const TB*>(p.bias.ptr) + b * p.bias.sb + h * p.bias.sh + k_ld;
+        if (!bias_matrix)
+            bias_vector = static_cast<float>(bias_col[0]) * kLog2e;
+        else if (tile_begin < ntiles)
+            bias_cur.load(bias_col, p.bias.sn, tile_begin * BQ + g * 16, p.Tq, (tile_begin + 1) * BQ <= p.Tq);
     }
 
     for (int j = tile_begin; j < ntiles; ++j) {
         const int buf = j & 1;
         const int q0 = j * BQ;
-        if (j + 1 < ntiles) issue_loads(j + 1);
-
+        if (j + 1 < ntiles) {
+            issue_loads(j + 1);
+            if constexpr (HAS_BIAS) {
+                if (bias_matrix) bias_nxt.load(bias_col, p.bias.sn, q0 + BQ + g * 16, p.Tq, q0 + 2 * BQ <= p.Tq);
+            }
+        }
         float bias_r[16];
         if constexpr (HAS_BIAS) {
-            if (p.bias_kind == RGD_BIAS_MATRIX) {
-                const bool rows_ok = q0 + BQ <= p.Tq;
-                const int qf = q0 + g * 16;
-                if (p.bias_dtype == RGD_BF16)
-                    load_bias_column<bf16_t>(bias_col, p.bias.sn, qf, p.Tq, rows_ok, bias_r);
-                else if (p.bias_dtype == RGD_F16)
-                    load_bias_column<f16_t>(bias_col, p.bias.sn, qf, p.Tq, rows_ok, bias_r);
-                else
-                    load_bias_column<float>(bias_col, p.bias.sn, qf, p.Tq, rows_ok, bias_r);
-            }
+            if (bias_matrix) bias_cur.decode(bias_r);
         }
 
         const T* qs = reinterpret_cast<const T*>(smem_raw + buf * BUFB);
@@ -472,7 +474,7 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dkv_
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             if constexpr (HAS_BIAS) {
-                const float bl = p.bias_kind == RGD_BIAS_VECTOR ? bias_vector + nlse[v] : fmaf(bias_r[v], kLog2e, nlse[v]);
+                const float bl = bias_matrix ? fmaf(bias_r[v], kLog2e, nlse[v]) : bias_vector + nlse[v];
                 s[v] = fmaf(s[v], p.scale_log2, bl);
             } else {
                 s[v] = fmaf(s[v], p.scale_log2, nlse[v]);
@@ -514,7 +516,12 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dkv_
                 dk_acc[d] = MM::run(as_v8<T>(qa), db, dk_acc[d]);
             }
         }
-        if (j + 1 < ntiles) store_tiles(buf ^ 1);
+        if (j + 1 < ntiles) {
+            store_tiles(buf ^ 1);
+            if constexpr (HAS_BIAS) {
+                if (bias_matrix) bias_cur = bias_nxt;
+            }
+        }
         __syncthreads();
     }
 

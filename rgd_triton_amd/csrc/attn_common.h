@@ -69,51 +69,46 @@ template <typename T> __device__ __forceinline__ uint32_t pack2(float lo, float 
     return __builtin_bit_cast(uint32_t, t);
 }
 
-// 16 contiguous bias values for one lane -> fp32, scaled by log2(e).  dtype is the bias element type.
-// `vec` = the run is 16-byte aligned and fully in range; otherwise elements >= limit read as 0.
-__device__ __forceinline__ void load_bias16(const void* base, int64_t off, int dtype, int first, int limit, bool vec,
-                                            float scale, float (&out)[16]) {
-    if (dtype == RGD_F32) {
-        const float* p = static_cast<const float*>(base) + off;
-        if (vec) {
+// Bias kinds of the kernel templates: no bias, bias stored in the tensor dtype T, bias stored in fp32.
+enum { BIAS_OFF = 0, BIAS_SAME = 1, BIAS_F32 = 2 };
+template <typename T, int BIAS> struct BiasElem { typedef T type; };
+template <typename T> struct BiasElem<T, BIAS_F32> { typedef float type; };
+
+// Raw bias of one lane for one 64-key tile in the "query per lane" layout: two runs of 16 contiguous
+// keys (key0 + 32*kb + 16*g ...).  load() only issues the memory reads, so it can run a whole tile
+// ahead of decode(); the registers hold the undecoded bits (8 VGPRs for a 16-bit bias).
+template <typename TB> struct BiasRuns {
+    static constexpr int NV = 16 * sizeof(TB) / 16;  // 16-byte vectors per run
+    u32x4 raw[2][NV];
+
+    // row: &bias[b, h, q, 0].  fast = the run is 16-byte aligned and all 64 keys of the tile exist.
+    __device__ __forceinline__ void load(const TB* __restrict__ row, int key0, int g, int Tk, bool fast) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                f32x4 t = *reinterpret_cast<const f32x4*>(p + first + 4 * i);
+        for (int kb = 0; kb < 2; ++kb) {
+            const int first = key0 + kb * 32 + g * 16;
+            if (fast) {
+                const u32x4* src = reinterpret_cast<const u32x4*>(row + first);
 #pragma unroll
-                for (int e = 0; e < 4; ++e) out[4 * i + e] = t[e] * scale;
-            }
-        } else {
-#pragma unroll
-            for (int e = 0; e < 16; ++e) out[e] = (first + e < limit) ? p[first + e] * scale : 0.f;
-        }
-    } else {
-        const uint16_t* p = static_cast<const uint16_t*>(base) + off;
-        Pack16 a, b;
-        if (vec) {
-            a.v = *reinterpret_cast<const u32x4*>(p + first);
-            b.v = *reinterpret_cast<const u32x4*>(p + first + 8);
-        } else {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                a.h[e] = (first + e < limit) ? p[first + e] : (uint16_t)0;
-                b.h[e] = (first + 8 + e < limit) ? p[first + 8 + e] : (uint16_t)0;
-            }
-        }
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            float x, y;
-            if (dtype == RGD_BF16) {
-                x = __builtin_bit_cast(float, (uint32_t)a.h[e] << 16);
-                y = __builtin_bit_cast(float, (uint32_t)b.h[e] << 16);
+                for (int i = 0; i < NV; ++i) raw[kb][i] = src[i];
             } else {
-                x = static_cast<float>(__builtin_bit_cast(f16_t, a.h[e]));
-                y = static_cast<float>(__builtin_bit_cast(f16_t, b.h[e]));
+                // element loads from clamped indices; keys >= Tk are masked by the caller
+                TB tmp[16];
+#pragma unroll
+                for (int e = 0; e < 16; ++e) tmp[e] = row[min(first + e, Tk - 1)];
+                __builtin_memcpy(&raw[kb][0], tmp, sizeof(tmp));
             }
-            out[e] = x * scale;
-            out[8 + e] = y * scale;
         }
     }
-}
+    __device__ __forceinline__ void decode(float (&out)[2][16]) const {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            TB tmp[16];
+            __builtin_memcpy(tmp, &raw[kb][0], sizeof(tmp));
+#pragma unroll
+            for (int e = 0; e < 16; ++e) out[kb][e] = static_cast<float>(tmp[e]);
+        }
+    }
+};
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 

@@ -42,8 +42,10 @@ template <int DPAD> struct AttnFwdSmem {
     static constexpr size_t BYTES = 2 * 2 * TILE * 2;  // K and V, double buffered
 };
 
-template <typename T, int DPAD, bool HAS_BIAS>
+template <typename T, int DPAD, int BIAS>
 __global__ __launch_bounds__(ATTN_THREADS, DPAD <= 64 ? 2 : 1) void attn_fwd_kernel(const AttnFwdParams p) {
+    constexpr bool HAS_BIAS = BIAS != BIAS_OFF;
+    typedef typename BiasElem<T, BIAS>::type TB;
     typedef Mfma<T> MM;
     typedef AttnFwdSmem<DPAD> SM;
     constexpr int ST = SM::ST;
@@ -146,26 +148,25 @@ __global__ __launch_bounds__(ATTN_THREADS, DPAD <= 64 ? 2 : 1) void attn_fwd_ker
     const int tr_off = ((lane & 15) >> 2) * ST + mfma_row_perm(((lane >> 4) & 1) * 16 + (lane & 3) * 4) +
                        g * 16 * ST;  // V^T via transposing reads: tile row (key) j, column quad
 
-    const char* bias_base = nullptr;
-    int64_t bias_row = 0;
+    // bias of this lane's query row, fetched one tile ahead of its use
+    const TB* bias_row = nullptr;
+    BiasRuns<TB> bias_cur, bias_nxt;
     if constexpr (HAS_BIAS) {
-        bias_base = static_cast<const char*>(p.bias.ptr);
-        bias_row = b * p.bias.sb + h * p.bias.sh + (int64_t)q_ld * p.bias.sn;
+        bias_row = static_cast<const TB*>(p.bias.ptr) + b * p.bias.sb + h * p.bias.sh + (int64_t)q_ld * p.bias.sn;
+        if (ntiles > 0) bias_cur.load(bias_row, 0, g, p.Tk, p.bias_vec && ATTN_BN <= p.Tk);
     }
 
     for (int j = 0; j < ntiles; ++j) {
         const int buf = j & 1;
         const int key0 = j * ATTN_BN;
-        if (j + 1 < ntiles) issue_loads(j + 1);
-
         const bool tail = key0 + ATTN_BN > p.Tk;
-        float bias_v[2][16];
-        if constexpr (HAS_BIAS) {
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-                load_bias16(bias_base, bias_row, p.bias_dtype, key0 + kb * 32 + g * 16, p.Tk, p.bias_vec && !tail, 1.0f,
-                            bias_v[kb]);
+        if (j + 1 < ntiles) {
+            issue_loads(j + 1);
+            if constexpr (HAS_BIAS)
+                bias_nxt.load(bias_row, key0 + ATTN_BN, g, p.Tk, p.bias_vec && key0 + 2 * ATTN_BN <= p.Tk);
         }
+        float bias_v[2][16];
+        if constexpr (HAS_BIAS) bias_cur.decode(bias_v);
 
         // ---- S^T = K . Q^T ----
         const T* ks = ks_base + buf * TILE + a_off;
@@ -258,7 +259,10 @@ __global__ __launch_bounds__(ATTN_THREADS, DPAD <= 64 ? 2 : 1) void attn_fwd_ker
             }
         }
 
-        if (j + 1 < ntiles) store_tiles(buf ^ 1);
+        if (j + 1 < ntiles) {
+            store_tiles(buf ^ 1);
+            if constexpr (HAS_BIAS) bias_cur = bias_nxt;
+        }
         __syncthreads();
     }
 
