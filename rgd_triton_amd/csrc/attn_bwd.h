@@ -87,8 +87,9 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dq_k
     T* const vs_base = ks_base + 2 * TILE;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 31, g = lane >> 5;
-    const int qb = blockIdx.x % p.nblk;
-    const int bh = blockIdx.x / p.nblk;
+    const int bid = xcd_remap(blockIdx.x, gridDim.x);
+    const int qb = bid % p.nblk;
+    const int bh = bid / p.nblk;
     const int b = bh / p.H, h = bh - b * p.H;
     const int q_row = qb * BWD_BM + wave * 32 + li;
     const bool q_valid = q_row < p.Tq;
@@ -317,8 +318,9 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dkv_
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 31, g = lane >> 5;
-    const int kblk = blockIdx.x % p.nblk;
-    const int bh = blockIdx.x / p.nblk;
+    const int bid = xcd_remap(blockIdx.x, gridDim.x);
+    const int kblk = bid % p.nblk;
+    const int bh = bid / p.nblk;
     const int b = bh / p.H, h = bh - b * p.H;
     const int key = kblk * BWD_BM + wave * 32 + li;  // this lane's key
     const bool k_valid = key < p.Tk;

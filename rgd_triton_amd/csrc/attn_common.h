@@ -148,6 +148,17 @@ template <> __device__ __forceinline__ float add_pair<f16_t>(uint32_t packed, fl
     return __builtin_amdgcn_fdot2(__builtin_bit_cast(V2, packed), ones, acc, false);
 }
 
+// Workgroup ids are handed to the 8 XCDs round-robin and every XCD has its own L2.  This maps the
+// hardware id to a logical id so that each XCD works through a contiguous range of logical ids:
+// workgroups that share K/V (same batch and head, neighbouring row blocks) then run on one XCD, one
+// after the other, and find those tiles in that XCD's L2.
+constexpr int kNumXcd = 8;
+__device__ __forceinline__ int xcd_remap(int id, int n) {
+    const int per = n / kNumXcd, rem = n % kNumXcd;
+    const int x = id % kNumXcd, slot = id / kNumXcd;
+    return x < rem ? x * (per + 1) + slot : rem * (per + 1) + (x - rem) * per + slot;
+}
+
 struct AttnTensor {
     const void* ptr;
     int64_t sb, sh, sn;

@@ -64,8 +64,9 @@ __global__ __launch_bounds__(ATTN_THREADS, DPAD <= 64 ? 2 : 1) void attn_fwd_ker
     const int li = lane & 31;
     const int g = lane >> 5;
 
-    const int qb = blockIdx.x % p.nqb;
-    const int bh = blockIdx.x / p.nqb;
+    const int bid = xcd_remap(blockIdx.x, gridDim.x);
+    const int qb = bid % p.nqb;
+    const int bh = bid / p.nqb;
     const int b = bh / p.H;
     const int h = bh - b * p.H;
 
