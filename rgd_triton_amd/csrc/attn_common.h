@@ -99,6 +99,12 @@ template <typename TB> struct BiasRuns {
             }
         }
     }
+    __device__ __forceinline__ void decode_run(int kb, float (&out)[16]) const {
+        TB tmp[16];
+        __builtin_memcpy(tmp, &raw[kb][0], sizeof(tmp));
+#pragma unroll
+        for (int e = 0; e < 16; ++e) out[e] = static_cast<float>(tmp[e]);
+    }
     __device__ __forceinline__ void decode(float (&out)[2][16]) const {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {

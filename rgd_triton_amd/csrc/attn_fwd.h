@@ -43,7 +43,7 @@ template <int DPAD> struct AttnFwdSmem {
 };
 
 template <typename T, int DPAD, int BIAS>
-__global__ __launch_bounds__(ATTN_THREADS, DPAD <= 64 ? 2 : 1) void attn_fwd_kernel(const AttnFwdParams p) {
+__global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 : 2) void attn_fwd_kernel(const AttnFwdParams p) {
     constexpr bool HAS_BIAS = BIAS != BIAS_OFF;
     typedef typename BiasElem<T, BIAS>::type TB;
     typedef Mfma<T> MM;
@@ -53,6 +53,10 @@ __global__ __launch_bounds__(ATTN_THREADS, DPAD <= 64 ? 2 : 1) void attn_fwd_ker
     constexpr int NC = DPAD / 16;   // d chunks of the first product
     constexpr int NDB = DPAD / 32;  // 32-row blocks of O^T
     constexpr int CPR = DPAD / 8;   // 16-byte chunks per K/V row
+    // d > 64: a 32-key half is finished (S -> p -> PV) before the next starts, which keeps only 16 logits
+    // live and lets two wavefronts share a SIMD; at d <= 64 three wavefronts fit either way and the joint
+    // form measured faster
+    constexpr bool SPLIT_HALVES = DPAD > 64;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     T* const ks_base = reinterpret_cast<T*>(smem_raw);
@@ -99,42 +103,44 @@ __global__ __launch_bounds__(ATTN_THREADS, DPAD <= 64 ? 2 : 1) void attn_fwd_ker
     constexpr int LOADS = TASKS / ATTN_THREADS;
     const T* kbase = static_cast<const T*>(p.k.ptr) + b * p.k.sb + h * p.k.sh;
     const T* vbase = static_cast<const T*>(p.v.ptr) + b * p.v.sb + h * p.v.sh;
-    int ld_key[LOADS], ld_dc[LOADS], koff[LOADS], voff[LOADS], soff[LOADS];
-#pragma unroll
-    for (int i = 0; i < LOADS; ++i) {
-        const int id = tid + i * ATTN_THREADS;
-        ld_key[i] = id / CPR;
-        ld_dc[i] = id % CPR;
-        koff[i] = ld_key[i] * (int)p.k.sn + ld_dc[i] * 8;
-        voff[i] = ld_key[i] * (int)p.v.sn + ld_dc[i] * 8;
-        soff[i] = ld_key[i] * ST + ld_dc[i] * 8;
-    }
+    // chunk i of this thread is row (ld_key0 + i*ROWS_PER_PASS) when the row length divides the
+    // workgroup size (head dims 32/64/128); otherwise (96) every chunk has its own row and column
+    constexpr bool REGULAR = ATTN_THREADS % CPR == 0;
+    constexpr int ROWS_PER_PASS = ATTN_THREADS / CPR;
+    const int ld_key0 = tid / CPR, ld_dc0 = tid % CPR;
+    auto chunk_key = [&](int i) { return REGULAR ? ld_key0 + i * ROWS_PER_PASS : (tid + i * ATTN_THREADS) / CPR; };
+    auto chunk_dc = [&](int i) { return REGULAR ? ld_dc0 : (tid + i * ATTN_THREADS) % CPR; };
+    const int koff0 = ld_key0 * (int)p.k.sn + ld_dc0 * 8;
+    const int voff0 = ld_key0 * (int)p.v.sn + ld_dc0 * 8;
     const bool fast_tiles = vec && p.D == DPAD;  // full rows, 16-byte loads: no masking except in the last tile
     u32x4 kst[LOADS], vst[LOADS];
     auto issue_loads = [&](int tile) {
         const int key0 = tile * ATTN_BN;
         const T* kt = kbase + (int64_t)key0 * p.k.sn;
         const T* vt = vbase + (int64_t)key0 * p.v.sn;
-        if (fast_tiles && key0 + ATTN_BN <= p.Tk) {
+        if (REGULAR && fast_tiles && key0 + ATTN_BN <= p.Tk) {
 #pragma unroll
             for (int i = 0; i < LOADS; ++i) {
-                kst[i] = *reinterpret_cast<const u32x4*>(kt + koff[i]);
-                vst[i] = *reinterpret_cast<const u32x4*>(vt + voff[i]);
+                // uniform part (tile base + i*ROWS_PER_PASS rows) + fixed per-thread offset
+                kst[i] = *reinterpret_cast<const u32x4*>(kt + (int64_t)(i * ROWS_PER_PASS) * p.k.sn + koff0);
+                vst[i] = *reinterpret_cast<const u32x4*>(vt + (int64_t)(i * ROWS_PER_PASS) * p.v.sn + voff0);
             }
         } else {
 #pragma unroll
             for (int i = 0; i < LOADS; ++i) {
-                const bool ok = key0 + ld_key[i] < p.Tk;
-                kst[i] = load8<T>(kt + (int64_t)ld_key[i] * p.k.sn, ld_dc[i] * 8, p.D, ok, vec);
-                vst[i] = load8<T>(vt + (int64_t)ld_key[i] * p.v.sn, ld_dc[i] * 8, p.D, ok, vec);
+                const int key = chunk_key(i), dc = chunk_dc(i);
+                const bool ok = key0 + key < p.Tk;
+                kst[i] = load8<T>(kt + (int64_t)key * p.k.sn, dc * 8, p.D, ok, vec);
+                vst[i] = load8<T>(vt + (int64_t)key * p.v.sn, dc * 8, p.D, ok, vec);
             }
         }
     };
     auto store_tiles = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < LOADS; ++i) {
-            *reinterpret_cast<u32x4*>(ks_base + buf * TILE + soff[i]) = kst[i];
-            *reinterpret_cast<u32x4*>(vs_base + buf * TILE + soff[i]) = vst[i];
+            const int so = chunk_key(i) * ST + chunk_dc(i) * 8;
+            *reinterpret_cast<u32x4*>(ks_base + buf * TILE + so) = kst[i];
+            *reinterpret_cast<u32x4*>(vs_base + buf * TILE + so) = vst[i];
         }
     };
 
@@ -166,97 +172,186 @@ __global__ __launch_bounds__(ATTN_THREADS, DPAD <= 64 ? 2 : 1) void attn_fwd_ker
             if constexpr (HAS_BIAS)
                 bias_nxt.load(bias_row, key0 + ATTN_BN, g, p.Tk, p.bias_vec && key0 + 2 * ATTN_BN <= p.Tk);
         }
-        float bias_v[2][16];
-        if constexpr (HAS_BIAS) bias_cur.decode(bias_v);
+        if constexpr (!SPLIT_HALVES) {
+            // d <= 64: both 32-key halves of the tile go through the softmax together
 
-        // ---- S^T = K . Q^T ----
-        const T* ks = ks_base + buf * TILE + a_off;
-        f32x16 s[2];
+            // ---- S^T = K . Q^T ----
+            const T* ks = ks_base + buf * TILE + a_off;
+            f32x16 s[2];
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
+            for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
-            for (int v = 0; v < 16; ++v) s[kb][v] = 0.f;
+                for (int v = 0; v < 16; ++v) s[kb][v] = 0.f;
 #pragma unroll
-            for (int c = 0; c < NC; ++c) {
-                const u32x4 a = *reinterpret_cast<const u32x4*>(ks + kb * 32 * ST + c * 16);
-                s[kb] = MM::run(as_v8<T>(a), qreg[c], s[kb]);
-            }
-        }
-
-        // ---- t = logit - m_ref (log2 domain) ----
-        const float m_off = m_ref == -INFINITY ? 0.f : m_ref;
-        float tmax = -INFINITY;
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                if constexpr (HAS_BIAS)
-                    s[kb][v] = fmaf(s[kb][v], p.scale_log2, fmaf(bias_v[kb][v], kLog2e, -m_off));
-                else
-                    s[kb][v] = fmaf(s[kb][v], p.scale_log2, -m_off);
-            }
-        const bool diag = p.causal && (key0 + ATTN_BN - 1 > qb * ATTN_BM + wave * 32);
-        if (tail || diag) {
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int key = key0 + kb * 32 + g * 16 + v;
-                    if (key >= p.Tk || (p.causal && key > q_row)) s[kb][v] = -INFINITY;
+                for (int c = 0; c < NC; ++c) {
+                    const u32x4 a = *reinterpret_cast<const u32x4*>(ks + kb * 32 * ST + c * 16);
+                    s[kb] = MM::run(as_v8<T>(a), qreg[c], s[kb]);
                 }
-        }
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int v = 0; v < 16; v += 2) tmax = fmaxf(fmaxf(tmax, s[kb][v]), s[kb][v + 1]);
-        tmax = fmaxf(tmax, lane_xor32(tmax));
+            }
 
-        // move the reference exponent only when needed (first finite logit of the row, or growth > 2^8)
-        const bool move = (m_ref == -INFINITY) ? (tmax != -INFINITY) : (tmax > ATTN_RESCALE_THRESHOLD);
-        if (__builtin_amdgcn_ballot_w64(move) != 0) {
-            const float shift = move ? tmax : 0.f;
-            const float alpha = move ? __builtin_amdgcn_exp2f(m_ref - (m_off + shift)) : 1.f;  // 0 when m_ref was -inf
-            m_ref = move ? m_off + shift : m_ref;
-            l_run *= alpha;
+            // ---- t = logit - m_ref (log2 domain) ----
+            const float m_off = m_ref == -INFINITY ? 0.f : m_ref;
+            float tmax = -INFINITY;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                if constexpr (HAS_BIAS) {
+                    float bias_v[16];
+                    bias_cur.decode_run(kb, bias_v);
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) s[kb][v] = fmaf(s[kb][v], p.scale_log2, fmaf(bias_v[v], kLog2e, -m_off));
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) s[kb][v] = fmaf(s[kb][v], p.scale_log2, -m_off);
+                }
+            }
+            const bool diag = p.causal && (key0 + ATTN_BN - 1 > qb * ATTN_BM + wave * 32);
+            if (tail || diag) {
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int key = key0 + kb * 32 + g * 16 + v;
+                        if (key >= p.Tk || (p.causal && key > q_row)) s[kb][v] = -INFINITY;
+                    }
+            }
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) s[kb][v] -= shift;
-#pragma unroll
-            for (int d = 0; d < NDB; ++d)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) oacc[d][v] *= alpha;
-        }
+                for (int v = 0; v < 16; v += 2) tmax = fmaxf(fmaxf(tmax, s[kb][v]), s[kb][v + 1]);
+            tmax = fmaxf(tmax, lane_xor32(tmax));
 
-        // ---- p = exp2(t), packed to the operand type ----
-        uint32_t pk[2][8];
-        float lsum0 = 0.f, lsum1 = 0.f;  // the row sum uses the unrounded fp32 values: LSE keeps fp32 accuracy
+            // move the reference exponent only when needed (first finite logit of the row, or growth > 2^8)
+            const bool move = (m_ref == -INFINITY) ? (tmax != -INFINITY) : (tmax > ATTN_RESCALE_THRESHOLD);
+            if (__builtin_amdgcn_ballot_w64(move) != 0) {
+                const float shift = move ? tmax : 0.f;
+                const float alpha = move ? __builtin_amdgcn_exp2f(m_ref - (m_off + shift)) : 1.f;  // 0 when m_ref was -inf
+                m_ref = move ? m_off + shift : m_ref;
+                l_run *= alpha;
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+                for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-            for (int v = 0; v < 16; v += 2) {
-                const float p0 = __builtin_amdgcn_exp2f(s[kb][v]);
-                const float p1 = __builtin_amdgcn_exp2f(s[kb][v + 1]);
-                pk[kb][v / 2] = pack2<T>(p0, p1);
-                lsum0 += p0;
-                lsum1 += p1;
+                    for (int v = 0; v < 16; ++v) s[kb][v] -= shift;
+#pragma unroll
+                for (int d = 0; d < NDB; ++d)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) oacc[d][v] *= alpha;
             }
-        l_run += lsum0 + lsum1;
 
-        // ---- O^T += V^T . P^T ----
-        const T* vs = vs_base + buf * TILE + tr_off;
+            // ---- p = exp2(t), packed to the operand type ----
+            uint32_t pk[2][8];
+            float lsum0 = 0.f, lsum1 = 0.f;  // the row sum uses the unrounded fp32 values: LSE keeps fp32 accuracy
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            const int kb = t >> 1, jj = t & 1;
-            const u32x4 praw = {pk[kb][jj * 4 + 0], pk[kb][jj * 4 + 1], pk[kb][jj * 4 + 2], pk[kb][jj * 4 + 3]};
-            const typename MM::V8 pb = as_v8<T>(praw);
+            for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-            for (int d = 0; d < NDB; ++d) {
-                const T* src = vs + (kb * 32 + jj * 8) * ST + d * 32;
-                const u32x2 lo = lds_read_tr<T>(src);
-                const u32x2 hi = lds_read_tr<T>(src + 4 * ST);
-                const u32x4 a = {lo[0], lo[1], hi[0], hi[1]};
-                oacc[d] = MM::run(as_v8<T>(a), pb, oacc[d]);
+                for (int v = 0; v < 16; v += 2) {
+                    const float p0 = __builtin_amdgcn_exp2f(s[kb][v]);
+                    const float p1 = __builtin_amdgcn_exp2f(s[kb][v + 1]);
+                    pk[kb][v / 2] = pack2<T>(p0, p1);
+                    lsum0 += p0;
+                    lsum1 += p1;
+                }
+            l_run += lsum0 + lsum1;
+
+            // ---- O^T += V^T . P^T ----
+            const T* vs = vs_base + buf * TILE + tr_off;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const int kb = t >> 1, jj = t & 1;
+                const u32x4 praw = {pk[kb][jj * 4 + 0], pk[kb][jj * 4 + 1], pk[kb][jj * 4 + 2], pk[kb][jj * 4 + 3]};
+                const typename MM::V8 pb = as_v8<T>(praw);
+#pragma unroll
+                for (int d = 0; d < NDB; ++d) {
+                    const T* src = vs + (kb * 32 + jj * 8) * ST + d * 32;
+                    const u32x2 lo = lds_read_tr<T>(src);
+                    const u32x2 hi = lds_read_tr<T>(src + 4 * ST);
+                    const u32x4 a = {lo[0], lo[1], hi[0], hi[1]};
+                    oacc[d] = MM::run(as_v8<T>(a), pb, oacc[d]);
+                }
+            }
+        } else {
+            // Each 32-key half of the tile is a complete softmax step of its own (S -> p -> PV), so only 16
+            // logits are live at a time; the register budget buys wavefronts per SIMD, and those hide the
+            // LDS and matrix-pipe latencies of one another.
+            const bool diag = p.causal && (key0 + ATTN_BN - 1 > qb * ATTN_BM + wave * 32);
+            const T* ks = ks_base + buf * TILE + a_off;
+            const T* vs = vs_base + buf * TILE + tr_off;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                // ---- S^T = K . Q^T ----
+                f32x16 s;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) s[v] = 0.f;
+#pragma unroll
+                for (int c = 0; c < NC; ++c) {
+                    const u32x4 a = *reinterpret_cast<const u32x4*>(ks + kb * 32 * ST + c * 16);
+                    s = MM::run(as_v8<T>(a), qreg[c], s);
+                }
+
+                // ---- t = logit - m_ref (log2 domain) ----
+                const float m_off = m_ref == -INFINITY ? 0.f : m_ref;
+                if constexpr (HAS_BIAS) {
+                    float bias_v[16];
+                    bias_cur.decode_run(kb, bias_v);
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) s[v] = fmaf(s[v], p.scale_log2, fmaf(bias_v[v], kLog2e, -m_off));
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) s[v] = fmaf(s[v], p.scale_log2, -m_off);
+                }
+                if (tail || diag) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int key = key0 + kb * 32 + g * 16 + v;
+                        if (key >= p.Tk || (p.causal && key > q_row)) s[v] = -INFINITY;
+                    }
+                }
+                float tmax = -INFINITY;
+#pragma unroll
+                for (int v = 0; v < 16; v += 2) tmax = fmaxf(fmaxf(tmax, s[v]), s[v + 1]);
+                tmax = fmaxf(tmax, lane_xor32(tmax));
+
+                // move the reference exponent only when needed (first finite logit of the row, or growth > 2^8)
+                const bool move = (m_ref == -INFINITY) ? (tmax != -INFINITY) : (tmax > ATTN_RESCALE_THRESHOLD);
+                if (__builtin_amdgcn_ballot_w64(move) != 0) {
+                    const float shift = move ? tmax : 0.f;
+                    const float alpha = move ? __builtin_amdgcn_exp2f(m_ref - (m_off + shift)) : 1.f;  // 0 when m_ref was -inf
+                    m_ref = move ? m_off + shift : m_ref;
+                    l_run *= alpha;
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) s[v] -= shift;
+#pragma unroll
+                    for (int d = 0; d < NDB; ++d)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) oacc[d][v] *= alpha;
+                }
+
+                // ---- p = exp2(t), packed to the operand type; fp32 row sum of the unrounded values ----
+                uint32_t pk[8];
+                float lsum0 = 0.f, lsum1 = 0.f;
+#pragma unroll
+                for (int v = 0; v < 16; v += 2) {
+                    const float p0 = __builtin_amdgcn_exp2f(s[v]);
+                    const float p1 = __builtin_amdgcn_exp2f(s[v + 1]);
+                    pk[v / 2] = pack2<T>(p0, p1);
+                    lsum0 += p0;
+                    lsum1 += p1;
+                }
+                l_run += lsum0 + lsum1;
+
+                // ---- O^T += V^T . P^T ----
+#pragma unroll
+                for (int jj = 0; jj < 2; ++jj) {
+                    const u32x4 praw = {pk[jj * 4 + 0], pk[jj * 4 + 1], pk[jj * 4 + 2], pk[jj * 4 + 3]};
+                    const typename MM::V8 pb = as_v8<T>(praw);
+#pragma unroll
+                    for (int d = 0; d < NDB; ++d) {
+                        const T* src = vs + (kb * 32 + jj * 8) * ST + d * 32;
+                        const u32x2 lo = lds_read_tr<T>(src);
+                        const u32x2 hi = lds_read_tr<T>(src + 4 * ST);
+                        const u32x4 a = {lo[0], lo[1], hi[0], hi[1]};
+                        oacc[d] = MM::run(as_v8<T>(a), pb, oacc[d]);
+                    }
+                }
             }
         }
 
