@@ -179,15 +179,17 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
             const T* ks = ks_base + buf * TILE + a_off;
             f32x16 s[2];
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
+            for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) s[kb][v] = 0.f;
+            // the two halves alternate, so consecutive matrix instructions never wait for each other's result
 #pragma unroll
-                for (int c = 0; c < NC; ++c) {
+            for (int c = 0; c < NC; ++c)
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb) {
                     const u32x4 a = *reinterpret_cast<const u32x4*>(ks + kb * 32 * ST + c * 16);
                     s[kb] = MM::run(as_v8<T>(a), qreg[c], s[kb]);
                 }
-            }
 
             // ---- t = logit - m_ref (log2 domain) ----
             const float m_off = m_ref == -INFINITY ? 0.f : m_ref;
