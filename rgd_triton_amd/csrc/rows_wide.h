@@ -42,10 +42,15 @@ struct WideParams {
     float eps;
 };
 
-template <typename T, int OP, bool BWD, int G, int NV, int VEC, bool VECTOR, int U, int NW>
+// WPR = wavefronts per row.  1: a row is owned by G <= 64 lanes of one wavefront.  4: a row is owned by
+// all 256 lanes of 4 wavefronts (G == 64), the row statistics are combined through LDS; used for rows
+// too wide to keep x, dy, w and the dw accumulators of one row in the registers of 64 lanes.
+template <typename T, int OP, bool BWD, int G, int NV, int VEC, bool VECTOR, int U, int NW, int WPR>
 __global__ __launch_bounds__(NW * 64) void wide_rows_kernel(const WideParams p) {
     extern __shared__ float s_dw[];
     __shared__ int s_last;
+    __shared__ float s_red[2][2][NW];  // [parity][statistic][wavefront]
+    static_assert(WPR == 1 || G == 64, "multi-wavefront rows use whole wavefronts");
 
     const int which = (int)blockIdx.x >= p.h[0].nchunks ? 1 : 0;
     const WideHalf& h = p.h[which];
@@ -55,12 +60,14 @@ __global__ __launch_bounds__(NW * 64) void wide_rows_kernel(const WideParams p) 
     const int r0 = chunk * p.rows_per_chunk;
     const int r1 = min(h.T, r0 + p.rows_per_chunk);
 
-    constexpr int GPW = 64 / G;  // row groups per wave
-    constexpr int NSLOT = NW * GPW;
+    constexpr int GPW = 64 / G;               // rows per wavefront at a time (WPR == 1)
+    constexpr int NSLOT = NW * GPW / WPR;     // rows the block works on at a time
+    constexpr int GL = G * WPR;               // lanes per row
     const int lane = lane_id();
     const int wave = threadIdx.x >> 6;
-    const int lg = lane % G;
-    const int slot = wave * GPW + lane / G;
+    const int wsub = wave % WPR;              // position of this wavefront inside its row group
+    const int lg = wsub * 64 + lane % G;      // lane index inside the row
+    const int slot = WPR == 1 ? wave * GPW + lane / G : wave / WPR;
 
     const T* xb = static_cast<const T*>(h.x) + (int64_t)b * h.sx_b;
     const T* db = BWD ? static_cast<const T*>(h.dy) + (int64_t)b * h.sd_b : nullptr;
@@ -74,48 +81,70 @@ __global__ __launch_bounds__(NW * 64) void wide_rows_kernel(const WideParams p) 
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
             if (VECTOR && h.w_vec)
-                load_chunk_dyn<VEC, VECTOR>(wp, h.w_dtype, (k * G + lg) * VEC, C, wv[k]);
+                load_chunk_dyn<VEC, VECTOR>(wp, h.w_dtype, (k * GL + lg) * VEC, C, wv[k]);
             else
-                load_chunk_dyn<VEC, false>(wp, h.w_dtype, (k * G + lg) * VEC, C, wv[k]);
+                load_chunk_dyn<VEC, false>(wp, h.w_dtype, (k * GL + lg) * VEC, C, wv[k]);
 #pragma unroll
             for (int e = 0; e < VEC; ++e) dwacc[k][e] = 0.f;
         }
     }
 
-    for (int rbase = r0 + slot; rbase < r1; rbase += NSLOT * U) {
-        float xv[U][NV][VEC];
-        float dv[U][NV][VEC];
+    // the trip count is the same for every wavefront of the block (rows past the end are masked), so the
+    // block-wide barriers of the multi-wavefront mode are reached by everyone
+    const int iters = (r1 - r0 + NSLOT * U - 1) / (NSLOT * U);
+    for (int it = 0; it < iters; ++it) {
+        const int rbase = r0 + slot + it * NSLOT * U;
+        Chunk<T, VEC, VECTOR> xc[U][NV], dc[U][NV];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int r = rbase + u * NSLOT;
-            const int lim = r < r1 ? C : 0;
+            const int r = min(rbase + u * NSLOT, r1 - 1);  // a row that exists; masked below if past the end
             const T* xr = xb + (int64_t)r * h.sx_n;
 #pragma unroll
-            for (int k = 0; k < NV; ++k) load_chunk<T, VEC, VECTOR>(xr, (k * G + lg) * VEC, lim, xv[u][k]);
+            for (int k = 0; k < NV; ++k) xc[u][k].load(xr, (k * GL + lg) * VEC, C);
             if constexpr (BWD) {
                 const T* dr = db + (int64_t)r * h.sd_n;
 #pragma unroll
-                for (int k = 0; k < NV; ++k) load_chunk<T, VEC, VECTOR>(dr, (k * G + lg) * VEC, lim, dv[u][k]);
+                for (int k = 0; k < NV; ++k) dc[u][k].load(dr, (k * GL + lg) * VEC, C);
             }
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int r = rbase + u * NSLOT;
             const int lim = r < r1 ? C : 0;
+            float xv[NV][VEC], dv[NV][VEC];
             float ss = 0.f, sd = 0.f;
 #pragma unroll
-            for (int k = 0; k < NV; ++k)
+            for (int k = 0; k < NV; ++k) {
+                xc[u][k].decode((k * GL + lg) * VEC, lim, xv[k]);
+                if constexpr (BWD) dc[u][k].decode((k * GL + lg) * VEC, lim, dv[k]);
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) {
-                    const float x = xv[u][k][e];
+                    const float x = xv[k][e];
                     ss += x * x;
                     if constexpr (BWD) {
-                        const float g = HAS_W ? dv[u][k][e] * wv[k][e] : dv[u][k][e];
-                        sd += x * g;
+                        const float gr = HAS_W ? dv[k][e] * wv[k][e] : dv[k][e];
+                        sd += x * gr;
                     }
                 }
+            }
             ss = group_reduce<G>(ss);
             if constexpr (BWD) sd = group_reduce<G>(sd);
+            if constexpr (WPR > 1) {
+                const int par = (it * U + u) & 1;
+                if (lane == 0) {
+                    s_red[par][0][wave] = ss;
+                    if constexpr (BWD) s_red[par][1][wave] = sd;
+                }
+                __syncthreads();
+                const int w0 = wave - wsub;
+                ss = 0.f;
+                sd = 0.f;
+#pragma unroll
+                for (int i = 0; i < WPR; ++i) {
+                    ss += s_red[par][0][w0 + i];
+                    if constexpr (BWD) sd += s_red[par][1][w0 + i];
+                }
+            }
             float rn;  // rrms or rlen
             if constexpr (OP == WIDE_RMS) {
                 rn = rsqrtf(ss * h.inv_c + p.eps);
@@ -128,8 +157,7 @@ __global__ __launch_bounds__(NW * 64) void wide_rows_kernel(const WideParams p) 
 #pragma unroll
                 for (int k = 0; k < NV; ++k)
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e)
-                        out[k][e] = HAS_W ? xv[u][k][e] * rn * wv[k][e] : xv[u][k][e] * rn;
+                    for (int e = 0; e < VEC; ++e) out[k][e] = HAS_W ? xv[k][e] * rn * wv[k][e] : xv[k][e] * rn;
             } else {
                 // inner = mean(xhat*dy*w) for RMSNorm, sum(xhat*dy) for L2
                 const float inner = OP == WIDE_RMS ? sd * rn * h.inv_c : sd * rn;
@@ -137,15 +165,15 @@ __global__ __launch_bounds__(NW * 64) void wide_rows_kernel(const WideParams p) 
                 for (int k = 0; k < NV; ++k)
 #pragma unroll
                     for (int e = 0; e < VEC; ++e) {
-                        const float xh = xv[u][k][e] * rn;
-                        const float g = HAS_W ? dv[u][k][e] * wv[k][e] : dv[u][k][e];
-                        out[k][e] = (g - xh * inner) * rn;
-                        if constexpr (HAS_W) dwacc[k][e] += xh * dv[u][k][e];
+                        const float xh = xv[k][e] * rn;
+                        const float gr = HAS_W ? dv[k][e] * wv[k][e] : dv[k][e];
+                        out[k][e] = (gr - xh * inner) * rn;
+                        if constexpr (HAS_W) dwacc[k][e] += xh * dv[k][e];
                     }
             }
-            T* yr = yb + (int64_t)r * h.sy_n;
+            T* yr = yb + (int64_t)min(r, r1 - 1) * h.sy_n;
 #pragma unroll
-            for (int k = 0; k < NV; ++k) store_chunk<T, VEC, VECTOR>(yr, (k * G + lg) * VEC, lim, out[k]);
+            for (int k = 0; k < NV; ++k) store_chunk<T, VEC, VECTOR>(yr, (k * GL + lg) * VEC, lim, out[k]);
         }
     }
 
@@ -155,17 +183,19 @@ __global__ __launch_bounds__(NW * 64) void wide_rows_kernel(const WideParams p) 
         for (int k = 0; k < NV; ++k)
 #pragma unroll
             for (int e = 0; e < VEC; ++e) dwacc[k][e] = cross_group_sum<G>(dwacc[k][e]);
+        // wavefront w covers the channels of row position (w % WPR); the first WPR wavefronts store, the
+        // others add, one wavefront at a time
         for (int wv_i = 0; wv_i < NW; ++wv_i) {
             if (wave == wv_i && lane < G) {
 #pragma unroll
                 for (int k = 0; k < NV; ++k)
 #pragma unroll
                     for (int e = 0; e < VEC; ++e) {
-                        const int c = (k * G + lg) * VEC + e;
-                        if (c < C) s_dw[c] = wv_i == 0 ? dwacc[k][e] : s_dw[c] + dwacc[k][e];
+                        const int c = (k * GL + lg) * VEC + e;
+                        if (c < C) s_dw[c] = wv_i < WPR ? dwacc[k][e] : s_dw[c] + dwacc[k][e];
                     }
             }
-            __syncthreads();
+            if (wv_i % WPR == WPR - 1) __syncthreads();
         }
 
         const int tree = h.w_shared ? 0 : b;
@@ -178,36 +208,45 @@ __global__ __launch_bounds__(NW * 64) void wide_rows_kernel(const WideParams p) 
         }
         float* tree_part = h.part + (int64_t)tree * h.tree_rows * C;
         int* tree_ctr = h.ctr + (int64_t)tree * h.tree_ctrs;
+        // Partial rows travel between blocks through agent-scope (write-through) stores and loads, and
+        // each block waits for its own stores to complete before it takes a ticket.  That is all the
+        // ordering the tree needs, and it avoids a release fence, which on this multi-XCD part would
+        // write back the whole L2 (full of freshly written dx) once per block.
         {
             float* mine = tree_part + (int64_t)(h.lvl_row_off[0] + idx) * C;
-            for (int c = threadIdx.x; c < C; c += NW * 64) mine[c] = s_dw[c];
+            for (int c = threadIdx.x; c < C; c += NW * 64)
+                __hip_atomic_store(mine + c, s_dw[c], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         for (int lvl = 0;; ++lvl) {
             const int g = idx / WIDE_FANIN;
             const int gs = min(WIDE_FANIN, n - g * WIDE_FANIN);
-            __threadfence();  // release this block's partial row
+            __builtin_amdgcn_s_waitcnt(0);  // this thread's partial-row stores have completed
             __syncthreads();
             if (threadIdx.x == 0) {
                 int* cp = tree_ctr + h.lvl_ctr_off[lvl] + g;
-                const int t = __hip_atomic_fetch_add(cp, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+                const int t = __hip_atomic_fetch_add(cp, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 const int last = (t == gs - 1);
                 if (last) __hip_atomic_store(cp, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 s_last = last;
             }
             __syncthreads();
             if (!s_last) return;  // block-uniform
-            __threadfence();      // acquire the siblings' rows
             const int ng = (n + WIDE_FANIN - 1) / WIDE_FANIN;
             const float* src = tree_part + (int64_t)(h.lvl_row_off[lvl] + g * WIDE_FANIN) * C;
             float* dst = tree_part + (int64_t)(h.lvl_row_off[lvl + 1] + g) * C;
             for (int c = threadIdx.x; c < C; c += NW * 64) {
+                float v[WIDE_FANIN];
+#pragma unroll
+                for (int j = 0; j < WIDE_FANIN; ++j)
+                    v[j] = j < gs ? __hip_atomic_load(src + (int64_t)j * C + c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                  : 0.f;
                 float acc = 0.f;
-                for (int j = 0; j < gs; ++j)
-                    acc += __hip_atomic_load(src + (int64_t)j * C + c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                for (int j = 0; j < WIDE_FANIN; ++j) acc += v[j];  // fixed order
                 if (ng == 1)
                     store_dyn(dw_row, h.w_dtype, c, acc);
                 else
-                    dst[c] = acc;
+                    __hip_atomic_store(dst + c, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
             if (ng == 1) return;
             idx = g;
@@ -237,7 +276,7 @@ int wide_workspace(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2, si
 struct WideConfig {
     int op;
     bool bwd;
-    int G, NV;
+    int G, NV, WPR;
     bool vector;
 };
 // compile-time launch shape shared by the kernel instantiations and the host-side grid computation

@@ -96,26 +96,38 @@ int wide_launch(const char* name, int op, bool bwd, int64_t B, const WideHalfArg
     cfg.vector = vector;
     const int vec = vector ? 16 / es : 2;
     const int64_t chunks = (maxC + vec - 1) / vec;
+    // elements of one row a lane may hold: x (+ dy) (+ w and the dw accumulators) all stay in registers
+    const int max_epl = has_w ? 32 : 64;
+    cfg.WPR = 1;
+    cfg.NV = 0;
     if (chunks <= 64) {
         cfg.G = std::max(4, pow2ceil((int)chunks));
         cfg.NV = 1;
     } else {
-        static const int allowed[] = {2, 3, 4, 6, 8, 12, 16};
-        const int64_t need = (chunks + 63) / 64;
         cfg.G = 64;
-        cfg.NV = 0;
-        for (int nv : allowed)
-            if (nv >= need) {
+        static const int allowed1[] = {2, 3, 4, 6, 8, 12, 16};
+        static const int allowed4[] = {1, 2, 3, 4, 6, 8, 12, 16};
+        const int64_t need1 = (chunks + 63) / 64, need4 = (chunks + 255) / 256;
+        for (int nv : allowed1)
+            if (nv >= need1 && nv * vec <= max_epl) {
                 cfg.NV = nv;
                 break;
             }
+        if (cfg.NV == 0) {  // too wide for one wavefront: four wavefronts share a row
+            cfg.WPR = 4;
+            for (int nv : allowed4)
+                if (nv >= need4 && nv * vec <= max_epl) {
+                    cfg.NV = nv;
+                    break;
+                }
+        }
         RGD_REQUIRE(cfg.NV != 0, RGD_ERR_UNSUPPORTED,
                     "%s: rows of %lld elements exceed the register-resident limit (%d)", name, (long long)maxC,
-                    64 * 16 * vec);
+                    256 * max_epl);
     }
     const int NW = wide_waves(op, bwd);
     const int U = wide_unroll(bwd, cfg.NV);
-    const int row_quantum = NW * (64 / cfg.G) * U;
+    const int row_quantum = NW * (64 / cfg.G) / cfg.WPR * U;
     const bool tree = has_w && bwd;
     const int64_t target = (int64_t)rgd_num_cus() * (tree ? DW_BLOCKS_PER_CU : BLOCKS_PER_CU);
     int64_t rpc = (total_rows + target - 1) / target;

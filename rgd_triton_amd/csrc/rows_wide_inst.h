@@ -5,19 +5,27 @@
 
 #include "rows_wide.h"
 
-template <typename T, int OP, bool BWD, int G, int NV, bool VECTOR>
+template <typename T, int OP, bool BWD, int G, int NV, bool VECTOR, int WPR>
 static int wide_launch_one(const WideParams& p, dim3 grid, size_t lds, hipStream_t s) {
     constexpr int VEC = VECTOR ? 16 / (int)sizeof(T) : 2;
     constexpr int U = wide_unroll(BWD, NV);
     constexpr int NW = wide_waves(OP, BWD);
-    hipLaunchKernelGGL((wide_rows_kernel<T, OP, BWD, G, NV, VEC, VECTOR, U, NW>), grid, dim3(NW * 64), lds, s, p);
-    return 0;
+    // the host never selects more elements per lane than this (they would not stay in registers)
+    if constexpr (NV * VEC <= (OP == WIDE_RMS ? 32 : 64)) {
+        hipLaunchKernelGGL((wide_rows_kernel<T, OP, BWD, G, NV, VEC, VECTOR, U, NW, WPR>), grid, dim3(NW * 64), lds, s,
+                           p);
+        return 0;
+    }
+    rgd_set_error("wide rows: %d elements per lane were not compiled", NV * VEC);
+    return RGD_ERR_UNSUPPORTED;
 }
 
 template <typename T, int OP, bool BWD, bool VECTOR>
 static int wide_dispatch_shape(const WideConfig& c, const WideParams& p, dim3 grid, size_t lds, hipStream_t s) {
 #define WIDE_CASE(g, nv) \
-    if (c.G == g && c.NV == nv) return wide_launch_one<T, OP, BWD, g, nv, VECTOR>(p, grid, lds, s);
+    if (c.WPR == 1 && c.G == g && c.NV == nv) return wide_launch_one<T, OP, BWD, g, nv, VECTOR, 1>(p, grid, lds, s);
+#define WIDE_CASE4(nv) \
+    if (c.WPR == 4 && c.G == 64 && c.NV == nv) return wide_launch_one<T, OP, BWD, 64, nv, VECTOR, 4>(p, grid, lds, s);
     WIDE_CASE(4, 1)
     WIDE_CASE(8, 1)
     WIDE_CASE(16, 1)
@@ -30,8 +38,17 @@ static int wide_dispatch_shape(const WideConfig& c, const WideParams& p, dim3 gr
     WIDE_CASE(64, 8)
     WIDE_CASE(64, 12)
     WIDE_CASE(64, 16)
+    WIDE_CASE4(1)
+    WIDE_CASE4(2)
+    WIDE_CASE4(3)
+    WIDE_CASE4(4)
+    WIDE_CASE4(6)
+    WIDE_CASE4(8)
+    WIDE_CASE4(12)
+    WIDE_CASE4(16)
 #undef WIDE_CASE
-    rgd_set_error("wide rows: no kernel for G=%d NV=%d", c.G, c.NV);
+#undef WIDE_CASE4
+    rgd_set_error("wide rows: no kernel for G=%d NV=%d WPR=%d", c.G, c.NV, c.WPR);
     return RGD_ERR_UNSUPPORTED;
 }
 

@@ -129,3 +129,28 @@ def test_operators_refuse_cpu_tensors():
         rgd.FusedHeadLayerNorm()(q, q)
     with pytest.raises(AssertionError):
         rgd.FlashAttention()(q.half(), q.half(), q.half())
+
+
+def test_reference_import_paths_alias():
+    """rgd_triton_amd.alias.install() makes the reference's import paths resolve to this package"""
+    import importlib
+    import sys
+
+    from rgd_triton_amd import alias
+
+    assert "rgd_triton" not in sys.modules
+    try:
+        names = alias.install()
+        assert "rgd_triton.ops" in names
+        from rgd_triton.ops import FlashAttention, FusedRMSNorm2  # noqa: F401
+        from rgd_triton.triton.flash_attn.flash_attn_triton_cached import flash_attn_func
+        from rgd_triton.triton.normalization.fused_rmsnorm_cached import triton_fused_rms_func_fn
+        from rgd_triton.triton.rope.fused_ln_rope_cached import triton_fused_ln_rope_fn
+        import rgd_triton_amd as rgd
+
+        assert flash_attn_func is rgd.flash_attn_func and triton_fused_rms_func_fn is rgd.triton_fused_rms_func_fn
+        assert triton_fused_ln_rope_fn is rgd.triton_fused_ln_rope_fn and FlashAttention is rgd.FlashAttention
+        assert importlib.import_module("rgd_triton.triton.rope.head_rope_cached").triton_rope_fn is rgd.triton_rope_fn
+    finally:
+        for k in [k for k in sys.modules if k == "rgd_triton" or k.startswith("rgd_triton.")]:
+            del sys.modules[k]

@@ -9,7 +9,7 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("C", [32, 63, 97, 122, 257, 384, 510, 740, 1023, 2048])
+@pytest.mark.parametrize("C", [32, 63, 97, 122, 257, 384, 510, 740, 1023, 2048, 4097, 6144, 16384])
 @pytest.mark.parametrize("T", [14, 200, 1024])
 def test_l2_norm(T, C, dtype):
     from rgd_triton_amd import triton_norm_func_fn

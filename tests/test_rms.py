@@ -39,6 +39,30 @@ def test_rms_norm(T, unique_bw, C, dtype):
     assert dw.shape == dw_ref.shape and dw.dtype == dw_ref.dtype
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("C", [2049, 3072, 5120, 6144, 8192])
+@pytest.mark.parametrize("unique_bw", [False, True])
+@pytest.mark.parametrize("T", [7, 300])
+def test_rms_norm_wide_rows(T, unique_bw, C, dtype):
+    """Rows wider than one wavefront keeps in registers: four wavefronts share a row.  Odd C takes the
+    unvectorised loads, whose limit is 4096 elements."""
+    B = 2
+    (y, dx, dw), (y_ref, dx_ref, dw_ref) = _run(B, T, C, dtype, unique_bw, seed=C + T)
+    assert_close(y, y_ref, dtype, "rms", "y")
+    assert_close(dx, dx_ref, dtype, "rms", "dx")
+    rows = T if unique_bw else B * T
+    assert_close(dw, dw_ref, dtype, "rms", "dw", atol_scale=3 * rows * C ** 0.5)
+
+
+def test_rms_too_wide_is_rejected():
+    from rgd_triton_amd import triton_rms_func_fn
+
+    x = torch.zeros(1, 4, 8192 + 8, device="cuda", dtype=torch.bfloat16)
+    w = torch.ones(8192 + 8, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="register-resident"):
+        triton_rms_func_fn(x, w, 1e-6)
+
+
 @pytest.mark.parametrize("T", [1, 3, 31, 97, 200, 1025])
 def test_rms_ragged_rows(T):
     (y, dx, dw), (y_ref, dx_ref, dw_ref) = _run(3, T, 384, torch.bfloat16, False)
@@ -87,7 +111,7 @@ def test_rms_strided_views():
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("C,T", [(384, 239), (1023, 113), (1536, 512)])
+@pytest.mark.parametrize("C,T", [(384, 239), (1023, 113), (1536, 512), (6144, 67)])
 def test_rms_deterministic(C, T, dtype):
     """The reference's race test (tests/test_rms.py:193-246): batch 60, repeated runs must give
     bit-identical y, dx and dw."""
