@@ -37,6 +37,10 @@ int check_common(const char* name, int64_t B, int64_t H, int64_t Tq, int64_t Tk,
         RGD_REQUIRE(bias && bias->ptr, RGD_ERR_INVALID, "%s: null bias", name);
         RGD_REQUIRE(bias_dtype == dtype || bias_dtype == RGD_F32, RGD_ERR_INVALID,
                     "%s: bias must have the dtype of q or fp32", name);
+        // the kernels address a bias row block as a 32-bit lane offset: 16 rows plus a key index
+        RGD_REQUIRE(bias_kind == RGD_BIAS_VECTOR || (bias->stride_n >= 0 && bias->stride_n < (int64_t(1) << 24)),
+                    RGD_ERR_UNSUPPORTED,
+                    "%s: bias row stride %lld is outside [0, 2^24)", name, (long long)bias->stride_n);
     }
     return RGD_OK;
 }

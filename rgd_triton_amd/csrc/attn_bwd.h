@@ -34,7 +34,7 @@ struct AttnBwdParams {
 };
 
 template <int DPAD> struct BwdTile {
-    static constexpr int S = DPAD + 8;  // row stride of every staged tile (elements)
+    static constexpr int S = attn_lds_stride(DPAD);  // row stride of every staged tile (elements)
 };
 
 // writes 16 contiguous columns (two 16-byte stores on the vector path) of one output row
@@ -73,6 +73,9 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dq_k
     typedef typename BiasElem<T, BIAS>::type TB;
     typedef Mfma<T> MM;
     constexpr int BN = DqSmem<DPAD>::BN;
+    // starting the dP accumulators from -delta takes 16 registers; the bias variants at two wavefronts per
+    // SIMD have none to spare and subtract delta per element instead
+    constexpr bool DP_INIT = BIAS == BIAS_OFF || DPAD > 64;
     constexpr int ST = BwdTile<DPAD>::S;
     constexpr int TILE = DqSmem<DPAD>::TILE;
     constexpr int NC = DPAD / 16;
@@ -117,6 +120,9 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dq_k
     // rows that do not exist, and rows whose logits are all -inf, get probability 0 everywhere
     const float neg_lse_l2 = (q_valid && lse != -INFINITY) ? -lse * kLog2e : -INFINITY;
     if (g == 0 && q_row < p.Tq_rounded) p.delta[(int64_t)bh * p.Tq_rounded + q_row] = q_valid ? delta : 0.f;
+    f32x16 dp_init;  // -delta in every element: what the dP accumulators start from
+#pragma unroll
+    for (int v = 0; v < 16; ++v) dp_init[v] = -delta;
 
     f32x16 acc[NDB];
 #pragma unroll
@@ -194,13 +200,17 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dq_k
         if constexpr (HAS_BIAS) bias_cur.decode(bias_v);
         const T* ks = ks_base + buf * TILE + a_off;
         const T* vs = vs_base + buf * TILE + a_off;
+        // the dP accumulators start from -delta, so that product comes out as dP - delta
         f32x16 s[2], dp[2];
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                s[kb][v] = 0.f;
-                dp[kb][v] = 0.f;
+            for (int v = 0; v < 16; ++v) s[kb][v] = 0.f;
+            if constexpr (DP_INIT) {
+                dp[kb] = dp_init;
+            } else {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) dp[kb][v] = 0.f;
             }
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
@@ -237,7 +247,10 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dq_k
             for (int v = 0; v < 16; v += 2) {
                 const float p0 = __builtin_amdgcn_exp2f(s[kb][v]);
                 const float p1 = __builtin_amdgcn_exp2f(s[kb][v + 1]);
-                dsk[kb][v / 2] = pack2<T>(p0 * (dp[kb][v] - delta), p1 * (dp[kb][v + 1] - delta));
+                if constexpr (DP_INIT)
+                    dsk[kb][v / 2] = pack2<T>(p0 * dp[kb][v], p1 * dp[kb][v + 1]);
+                else
+                    dsk[kb][v / 2] = pack2<T>(p0 * (dp[kb][v] - delta), p1 * (dp[kb][v + 1] - delta));
             }
         // dQ^T += K^T . dS^T
         const T* kt = ks_base + buf * TILE + tr_off;
@@ -272,26 +285,41 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dq_k
 // ------------------------------------------------------------------------------------------------
 // dK / dV kernel
 // ------------------------------------------------------------------------------------------------
-template <int DPAD> struct DkvSmem {
-    static constexpr int BQ = 32;  // query rows per tile
+#ifndef RGD_DKV_OCC
+#define RGD_DKV_OCC 2  // wavefronts per SIMD of the dK/dV kernel without bias at head dims <= 64
+#endif
+#ifndef RGD_DKV_NSUB
+#define RGD_DKV_NSUB 2
+#endif
+// Query rows per loop iteration of the dK/dV kernel = 32 * dkv_nsub: each wavefront works on dkv_nsub
+// independent 32-row sub-tiles between two barriers, which gives the scheduler matrix work of one sub-tile
+// to put beside the exponentials of the other.  A bias costs the registers that would take.
+constexpr int dkv_nsub(int dpad, int bias) { return (bias == BIAS_OFF || dpad > 64) ? RGD_DKV_NSUB : 1; }
+template <int DPAD, int NSUB> struct DkvSmem {
+    static constexpr int BQ = 32 * NSUB;  // query rows per tile
     static constexpr int TILE = BQ * BwdTile<DPAD>::S;
-    // per buffer: Q tile, dO tile, then BQ floats of -lse*log2e and BQ floats of delta
+    // per buffer: Q tile, dO tile, then BQ floats of -lse*log2e and BQ floats of -delta
     static constexpr int BUF_BYTES = 2 * TILE * 2 + 2 * BQ * 4;
     static constexpr size_t BYTES = 2 * BUF_BYTES;
 };
 
-// 16 bias values of one key column (rows q_first .. +15 of the bias matrix) in the "key per lane"
-// layout.  load() only issues the reads so it can run a tile ahead of decode().
-// `rows_ok` = all 16 rows exist; otherwise rows >= Tq read the last existing row (masked out later).
+// 16 bias values of one key column (16 consecutive rows of the bias matrix) in the "key per lane" layout.
+// load() only issues the reads so it can run a tile ahead of decode().  `tile_rows` points at the first
+// bias row of the query tile and is the same for the whole wavefront, `lane_off` is this lane's element
+// offset from there (its key column plus 16*g rows), so every read is a wavefront-uniform base plus a
+// 32-bit lane offset and needs no per-lane address arithmetic.  A ragged last tile (rows_ok false) reads
+// the last existing row instead of rows >= Tq; the caller masks those.
 template <typename TB> struct BiasColumn {
     TB raw[16];
-    __device__ __forceinline__ void load(const TB* __restrict__ col, int64_t sn, int q_first, int Tq, bool rows_ok) {
+    __device__ __forceinline__ void load(const TB* __restrict__ tile_rows, int64_t sn, uint32_t lane_off, int row0,
+                                         int Tq, bool rows_ok) {
         if (rows_ok) {
 #pragma unroll
-            for (int v = 0; v < 16; ++v) raw[v] = col[(int64_t)(q_first + v) * sn];
+            for (int v = 0; v < 16; ++v) raw[v] = (tile_rows + v * sn)[lane_off];
         } else {
+            const TB* col = tile_rows + lane_off;  // rows_ok is false at most once per workgroup
 #pragma unroll
-            for (int v = 0; v < 16; ++v) raw[v] = col[(int64_t)min(q_first + v, Tq - 1) * sn];
+            for (int v = 0; v < 16; ++v) raw[v] = col[(int64_t)(min(row0 + v, Tq - 1) - row0) * sn];
         }
     }
     __device__ __forceinline__ void decode(float (&out)[16]) const {
@@ -301,18 +329,20 @@ template <typename TB> struct BiasColumn {
 };
 
 template <typename T, int DPAD, int BIAS>
-__global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dkv_kernel(const AttnBwdParams p) {
+__global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_DKV_OCC : 2) : 1) void attn_bwd_dkv_kernel(const AttnBwdParams p) {
     constexpr bool HAS_BIAS = BIAS != BIAS_OFF;
     typedef typename BiasElem<T, BIAS>::type TB;
     typedef Mfma<T> MM;
-    constexpr int BQ = DkvSmem<DPAD>::BQ;
+    constexpr int NSUB = dkv_nsub(DPAD, BIAS);
+    typedef DkvSmem<DPAD, NSUB> SM;
+    constexpr int BQ = SM::BQ;
     constexpr int ST = BwdTile<DPAD>::S;
-    constexpr int TILE = DkvSmem<DPAD>::TILE;
-    constexpr int BUFB = DkvSmem<DPAD>::BUF_BYTES;
+    constexpr int TILE = SM::TILE;
+    constexpr int BUFB = SM::BUF_BYTES;
     constexpr int NC = DPAD / 16;
     constexpr int NDB = DPAD / 32;
     constexpr int CPR = DPAD / 8;
-    constexpr int TASKS = BQ * CPR;  // 16-byte chunks of one tile: 128 .. 512
+    constexpr int TASKS = BQ * CPR;  // 16-byte chunks of one tile: 128 .. 1024
     constexpr int LOADS = (TASKS + BWD_THREADS - 1) / BWD_THREADS;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -391,7 +421,7 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dkv_
             const float l = lsep[ok ? q : 0];
             // rows that do not exist or have no finite logit get probability 0 (exp2(-inf))
             lse_st = (ok && l != -INFINITY) ? -l * kLog2e : -INFINITY;
-            delta_st = ok ? deltap[q] : 0.f;
+            delta_st = ok ? -deltap[q] : 0.f;  // negated: it is what the dP accumulator starts from
         }
     };
     auto store_tiles = [&](int buf) {
@@ -419,109 +449,119 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dkv_
     const int a_off = mfma_row_perm(li) * ST + g * 8;
     const int tr_off = ((lane & 15) >> 2) * ST + mfma_row_perm(((lane >> 4) & 1) * 16 + (lane & 3) * 4) + g * 16 * ST;
 
-    const TB* bias_col = nullptr;  // this lane's key column of the bias
-    float bias_vector = 0.f;
-    const bool bias_matrix = HAS_BIAS && p.bias_kind == RGD_BIAS_MATRIX;
-    BiasColumn<TB> bias_cur, bias_nxt;  // fetched one tile ahead of use
+    // A vector bias arrives with row stride 0, so it reads like a matrix whose rows are all the same.
+    const TB* bias_base = nullptr;  // bias of this batch and head (wavefront-uniform)
+    uint32_t bias_lane_off = 0;     // this lane's key column, 16*g rows down
+    BiasColumn<TB> bias_cur[NSUB], bias_nxt[NSUB];  // fetched one tile ahead of use
+    auto bias_load = [&](BiasColumn<TB> (&dst)[NSUB], int tile) {
+#pragma unroll
+        for (int u = 0; u < NSUB; ++u) {
+            const int q0 = tile * BQ + u * 32;
+            // the ragged sub-tile clamps rows per lane half: its row base is that of the lane's own first row
+            dst[u].load(bias_base + (int64_t)q0 * p.bias.sn, p.bias.sn, bias_lane_off, q0 + g * 16, p.Tq,
+                        q0 + 32 <= p.Tq);
+        }
+    };
     if constexpr (HAS_BIAS) {
-        bias_col = static_cast<const TB*>(p.bias.ptr) + b * p.bias.sb + h * p.bias.sh + k_ld;
-        if (!bias_matrix)
-            bias_vector = static_cast<float>(bias_col[0]) * kLog2e;
-        else if (tile_begin < ntiles)
-            bias_cur.load(bias_col, p.bias.sn, tile_begin * BQ + g * 16, p.Tq, (tile_begin + 1) * BQ <= p.Tq);
+        bias_base = static_cast<const TB*>(p.bias.ptr) + b * p.bias.sb + h * p.bias.sh;
+        bias_lane_off = (uint32_t)k_ld + (uint32_t)(g * 16) * (uint32_t)p.bias.sn;
+        if (tile_begin < ntiles) bias_load(bias_cur, tile_begin);
     }
 
     for (int j = tile_begin; j < ntiles; ++j) {
         const int buf = j & 1;
-        const int q0 = j * BQ;
         if (j + 1 < ntiles) {
             issue_loads(j + 1);
-            if constexpr (HAS_BIAS) {
-                if (bias_matrix) bias_nxt.load(bias_col, p.bias.sn, q0 + BQ + g * 16, p.Tq, q0 + 2 * BQ <= p.Tq);
-            }
+            if constexpr (HAS_BIAS) bias_load(bias_nxt, j + 1);
         }
-        float bias_r[16];
-        if constexpr (HAS_BIAS) {
-            if (bias_matrix) bias_cur.decode(bias_r);
-        }
-
         const T* qs = reinterpret_cast<const T*>(smem_raw + buf * BUFB);
         const T* dos = qs + TILE;
         const float* st = reinterpret_cast<const float*>(smem_raw + buf * BUFB + 2 * TILE * 2);
 
-        f32x16 s, dp;
+        // the dP accumulators start from -delta of their query rows, so that product comes out as dP - delta
+        f32x16 s[NSUB], dp[NSUB];
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            s[v] = 0.f;
-            dp[v] = 0.f;
-        }
+        for (int u = 0; u < NSUB; ++u)
 #pragma unroll
-        for (int c = 0; c < NC; ++c) {
-            const u32x4 qa = *reinterpret_cast<const u32x4*>(qs + a_off + c * 16);
-            s = MM::run(as_v8<T>(qa), kreg[c], s);
-            const u32x4 da = *reinterpret_cast<const u32x4*>(dos + a_off + c * 16);
-            dp = MM::run(as_v8<T>(da), vreg[c], dp);
-        }
-        float nlse[16], dlt[16];
+            for (int i = 0; i < 4; ++i) {
+                const f32x4 c = *reinterpret_cast<const f32x4*>(st + BQ + u * 32 + g * 16 + 4 * i);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const f32x4 a = *reinterpret_cast<const f32x4*>(st + g * 16 + 4 * i);
-            const f32x4 c = *reinterpret_cast<const f32x4*>(st + BQ + g * 16 + 4 * i);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                nlse[4 * i + e] = a[e];
-                dlt[4 * i + e] = c[e];
+                for (int e = 0; e < 4; ++e) {
+                    s[u][4 * i + e] = 0.f;
+                    dp[u][4 * i + e] = c[e];
+                }
             }
-        }
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
+        for (int c = 0; c < NC; ++c)
+#pragma unroll
+            for (int u = 0; u < NSUB; ++u) {
+                const u32x4 qa = *reinterpret_cast<const u32x4*>(qs + u * 32 * ST + a_off + c * 16);
+                s[u] = MM::run(as_v8<T>(qa), kreg[c], s[u]);
+                const u32x4 da = *reinterpret_cast<const u32x4*>(dos + u * 32 * ST + a_off + c * 16);
+                dp[u] = MM::run(as_v8<T>(da), vreg[c], dp[u]);
+            }
+#pragma unroll
+        for (int u = 0; u < NSUB; ++u) {
+            const int q0 = j * BQ + u * 32;
+            // t = logit - lse (log2 domain)
+            float nlse[16];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const f32x4 a = *reinterpret_cast<const f32x4*>(st + u * 32 + g * 16 + 4 * i);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) nlse[4 * i + e] = a[e];
+            }
             if constexpr (HAS_BIAS) {
-                const float bl = bias_matrix ? fmaf(bias_r[v], kLog2e, nlse[v]) : bias_vector + nlse[v];
-                s[v] = fmaf(s[v], p.scale_log2, bl);
+                float bias_r[16];
+                bias_cur[u].decode(bias_r);
+#pragma unroll
+                for (int v = 0; v < 16; ++v) s[u][v] = fmaf(s[u][v], p.scale_log2, fmaf(bias_r[v], kLog2e, nlse[v]));
             } else {
-                s[v] = fmaf(s[v], p.scale_log2, nlse[v]);
+#pragma unroll
+                for (int v = 0; v < 16; ++v) s[u][v] = fmaf(s[u][v], p.scale_log2, nlse[v]);
             }
-        }
-        const bool diag = p.causal && (q0 < kblk * BWD_BM + wave * 32 + 32);
-        if (!k_valid || diag) {
+            const bool diag = p.causal && (q0 < kblk * BWD_BM + wave * 32 + 32);
+            if (!k_valid || diag) {
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int q = q0 + g * 16 + v;
-                if (!k_valid || key > q) s[v] = -INFINITY;
+                for (int v = 0; v < 16; ++v) {
+                    const int q = q0 + g * 16 + v;
+                    if (!k_valid || key > q) s[u][v] = -INFINITY;
+                }
             }
-        }
-        uint32_t pk[8], dsk[8];
+            uint32_t pk[8], dsk[8];
 #pragma unroll
-        for (int v = 0; v < 16; v += 2) {
-            const float p0 = __builtin_amdgcn_exp2f(s[v]);
-            const float p1 = __builtin_amdgcn_exp2f(s[v + 1]);
-            pk[v / 2] = pack2<T>(p0, p1);
-            dsk[v / 2] = pack2<T>(p0 * (dp[v] - dlt[v]), p1 * (dp[v + 1] - dlt[v + 1]));
-        }
-        // dV^T += dO^T . P ;  dK^T += Q^T . dS
+            for (int v = 0; v < 16; v += 2) {
+                const float p0 = __builtin_amdgcn_exp2f(s[u][v]);
+                const float p1 = __builtin_amdgcn_exp2f(s[u][v + 1]);
+                pk[v / 2] = pack2<T>(p0, p1);
+                dsk[v / 2] = pack2<T>(p0 * dp[u][v], p1 * dp[u][v + 1]);
+            }
+            // dV^T += dO^T . P ;  dK^T += Q^T . dS
 #pragma unroll
-        for (int jj = 0; jj < 2; ++jj) {
-            const u32x4 praw = {pk[jj * 4 + 0], pk[jj * 4 + 1], pk[jj * 4 + 2], pk[jj * 4 + 3]};
-            const u32x4 draw = {dsk[jj * 4 + 0], dsk[jj * 4 + 1], dsk[jj * 4 + 2], dsk[jj * 4 + 3]};
-            const typename MM::V8 pb = as_v8<T>(praw), db = as_v8<T>(draw);
+            for (int jj = 0; jj < 2; ++jj) {
+                const u32x4 praw = {pk[jj * 4 + 0], pk[jj * 4 + 1], pk[jj * 4 + 2], pk[jj * 4 + 3]};
+                const u32x4 draw = {dsk[jj * 4 + 0], dsk[jj * 4 + 1], dsk[jj * 4 + 2], dsk[jj * 4 + 3]};
+                const typename MM::V8 pb = as_v8<T>(praw), db = as_v8<T>(draw);
 #pragma unroll
-            for (int d = 0; d < NDB; ++d) {
-                const T* dsrc = dos + tr_off + jj * 8 * ST + d * 32;
-                const u32x2 dlo = lds_read_tr<T>(dsrc);
-                const u32x2 dhi = lds_read_tr<T>(dsrc + 4 * ST);
-                const u32x4 da = {dlo[0], dlo[1], dhi[0], dhi[1]};
-                dv_acc[d] = MM::run(as_v8<T>(da), pb, dv_acc[d]);
-                const T* qsrc = qs + tr_off + jj * 8 * ST + d * 32;
-                const u32x2 qlo = lds_read_tr<T>(qsrc);
-                const u32x2 qhi = lds_read_tr<T>(qsrc + 4 * ST);
-                const u32x4 qa = {qlo[0], qlo[1], qhi[0], qhi[1]};
-                dk_acc[d] = MM::run(as_v8<T>(qa), db, dk_acc[d]);
+                for (int d = 0; d < NDB; ++d) {
+                    const T* dsrc = dos + u * 32 * ST + tr_off + jj * 8 * ST + d * 32;
+                    const u32x2 dlo = lds_read_tr<T>(dsrc);
+                    const u32x2 dhi = lds_read_tr<T>(dsrc + 4 * ST);
+                    const u32x4 da = {dlo[0], dlo[1], dhi[0], dhi[1]};
+                    dv_acc[d] = MM::run(as_v8<T>(da), pb, dv_acc[d]);
+                    const T* qsrc = qs + u * 32 * ST + tr_off + jj * 8 * ST + d * 32;
+                    const u32x2 qlo = lds_read_tr<T>(qsrc);
+                    const u32x2 qhi = lds_read_tr<T>(qsrc + 4 * ST);
+                    const u32x4 qa = {qlo[0], qlo[1], qhi[0], qhi[1]};
+                    dk_acc[d] = MM::run(as_v8<T>(qa), db, dk_acc[d]);
+                }
             }
         }
         if (j + 1 < ntiles) {
             store_tiles(buf ^ 1);
             if constexpr (HAS_BIAS) {
-                if (bias_matrix) bias_cur = bias_nxt;
+#pragma unroll
+                for (int u = 0; u < NSUB; ++u) bias_cur[u] = bias_nxt[u];
             }
         }
         __syncthreads();

@@ -14,6 +14,11 @@
 
 #include "common.h"
 
+// Row stride (elements) of the 16-bit tiles staged in LDS.  Measured on gfx950: with these strides both the
+// 16-byte row reads of the MFMA A operands and the transposing 8-byte reads run at the full LDS rate;
+// DPAD + 8 does too except for DPAD = 128, where the transposing reads take two-way bank conflicts.
+constexpr int attn_lds_stride(int dpad) { return dpad + (dpad == 128 ? 24 : 8); }
+
 template <typename T> struct Mfma;
 template <> struct Mfma<bf16_t> {
     typedef bf16x8 V8;

@@ -37,7 +37,7 @@ struct AttnFwdParams {
 };
 
 template <int DPAD> struct AttnFwdSmem {
-    static constexpr int ST = DPAD + 8;  // row stride of the K and V tiles (elements)
+    static constexpr int ST = attn_lds_stride(DPAD);  // row stride of the K and V tiles (elements)
     static constexpr int TILE = ATTN_BN * ST;
     static constexpr size_t BYTES = 2 * 2 * TILE * 2;  // K and V, double buffered
 };

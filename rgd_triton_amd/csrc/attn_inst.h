@@ -38,7 +38,7 @@ template <typename T> int dispatch_fwd(const AttnFwdParams& p, unsigned grid, hi
 
 template <typename T, int DPAD, int BIAS, bool DQ> int launch_bwd(const AttnBwdParams& p, unsigned grid, hipStream_t s) {
     auto kern = DQ ? attn_bwd_dq_kernel<T, DPAD, BIAS> : attn_bwd_dkv_kernel<T, DPAD, BIAS>;
-    constexpr size_t lds = DQ ? DqSmem<DPAD>::BYTES : DkvSmem<DPAD>::BYTES;
+    constexpr size_t lds = DQ ? DqSmem<DPAD>::BYTES : DkvSmem<DPAD, dkv_nsub(DPAD, BIAS)>::BYTES;
     static bool configured = false;
     if (!configured && lds > 48 * 1024) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
