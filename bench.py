@@ -32,7 +32,11 @@ MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # this file (profiles/), scaled by a copy kernel of known size; None until measured for a workload.
-MEASURED_TRAFFIC = {}
+MEASURED_TRAFFIC = {
+    # FETCH_SIZE 65767.0 KiB x 2.0 (copy calibration) + WRITE_SIZE 65536.0 KiB x 1.0, per launch of the
+    # LN+RoPE backward on this workload (profiles/head_rows_lnrope_config2.md)
+    "ln_rope_bwd_c2": 201799680,
+}
 
 
 def parse():
@@ -212,19 +216,112 @@ def attention_case(torch, name, B, T, H, D, dtype, bias_kind, iters=20):
             "bwd_tflops": round(flops * 10 / 14 / b_ms / 1e9, 2), "frac_mfma_peak": round(flops / tot / 1e9 / MFMA_PEAK_TFLOPS, 4)}
 
 
-def rows_case(torch, name, make, nbytes, nsets=4, iters=40):
-    """HBM-bound operator through the Module API + autograd, rotating buffer sets"""
-    sets = [make(i) for i in range(nsets)]
-    idx = [0]
+def time_pair(torch, fwd, bwd, nsets, iters=60, warmup=8):
+    """average ms of fwd(i) and of bwd(i) (i = buffer set), each timed as a run of back-to-back launches"""
+    out = []
+    for fn in (fwd, bwd):
+        for i in range(warmup):
+            fn(i % nsets)
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for i in range(iters):
+            fn(i % nsets)
+        b.record()
+        torch.cuda.synchronize()
+        out.append(a.elapsed_time(b) / iters)
+    return out
 
-    def run():
-        s = sets[idx[0] % nsets]
-        idx[0] += 1
-        s()
 
-    ms = time_api(torch, run, iters, 8)
-    return {"workload": name, "ms": round(ms, 4), "gbs": round(nbytes / ms / 1e6, 1),
-            "frac_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4), "path": "Module API + autograd (eager launches)"}
+def rows_result(torch, name, fwd, bwd, fwd_bytes, bwd_bytes, nsets, api=None):
+    """HBM-bound operator through the C ABI on rotating buffer sets (algorithmic bytes: every tensor read or
+    written once); `api` optionally times the same step through the Module API + autograd."""
+    f_ms, b_ms = time_pair(torch, fwd, bwd, nsets)
+    tot = f_ms + b_ms
+    r = {"workload": name, "fwd_us": round(f_ms * 1e3, 2), "bwd_us": round(b_ms * 1e3, 2),
+         "fwd_gbs": round(fwd_bytes / f_ms / 1e6, 1), "bwd_gbs": round(bwd_bytes / b_ms / 1e6, 1),
+         "gbs": round((fwd_bytes + bwd_bytes) / tot / 1e6, 1),
+         "frac_hbm_peak": round((fwd_bytes + bwd_bytes) / tot / 1e6 / HBM_PEAK_GBS, 4), "path": "C ABI, back-to-back launches"}
+    if api is not None:
+        r["module_api_ms"] = round(time_api(torch, api, 30, 5), 4)
+    return r
+
+
+def rms_case(torch, name, B, shapes, dtype, nsets, with_api=True):
+    """FusedRMSNorm (one shape) or FusedRMSNorm2 (two shapes) forward+backward, shared (C,) weights"""
+    import rgd_triton_amd as rgd
+    from rgd_triton_amd import _hip
+
+    lib, t3 = _hip.lib(), _hip.t3
+    code = _hip.dtype_code(dtype)
+    es = torch.empty(0, dtype=dtype).element_size()
+    st = _hip.stream_ptr(torch.device("cuda"))
+    (T1, C1), (T2, C2) = shapes[0], (shapes[1] if len(shapes) > 1 else (0, 0))
+    mk = lambda T, C: [torch.randn(B, T, C, device="cuda").to(dtype) for _ in range(nsets)]
+    x1, d1, x2, d2 = mk(T1, C1), mk(T1, C1), mk(T2, max(C2, 1)), mk(T2, max(C2, 1))
+    y1, y2 = [torch.empty_like(t) for t in x1], [torch.empty_like(t) for t in x2]
+    w1 = (1 + 0.1 * torch.randn(C1, device="cuda")).to(dtype)
+    w2 = (1 + 0.1 * torch.randn(max(C2, 1), device="cuda")).to(dtype)
+    dw1, dw2 = torch.empty_like(w1), torch.empty_like(w2)
+    ws, ct = ctypes.c_size_t(), ctypes.c_size_t()
+    assert lib.rgd_rms_bwd_workspace(B, T1, C1, T2, C2, ctypes.byref(ws), ctypes.byref(ct)) == 0
+    wbuf = torch.empty(max(ws.value, 1), dtype=torch.uint8, device="cuda")
+    cbuf = torch.zeros(max(ct.value, 1), dtype=torch.uint8, device="cuda")
+    if T2 == 0:
+        def fwd(i):
+            assert lib.rgd_rms_fwd(B, T1, C1, t3(x1[i]), t3(w1, 0), t3(y1[i]), code, code, 1e-6, st) == 0, lib.rgd_last_error()
+
+        def bwd(i):
+            assert lib.rgd_rms_bwd(B, T1, C1, t3(d1[i]), t3(x1[i]), t3(w1, 0), t3(y1[i]), t3(dw1, 0), 1, code, code, 1e-6,
+                                   wbuf.data_ptr(), ws.value, cbuf.data_ptr(), ct.value, st) == 0, lib.rgd_last_error()
+    else:
+        def fwd(i):
+            assert lib.rgd_fused_rms_fwd(B, T1, C1, T2, C2, t3(x1[i]), t3(w1, 0), t3(y1[i]), t3(x2[i]), t3(w2, 0), t3(y2[i]),
+                                         code, code, code, 1e-6, st) == 0, lib.rgd_last_error()
+
+        def bwd(i):
+            assert lib.rgd_fused_rms_bwd(B, T1, C1, T2, C2, t3(d1[i]), t3(x1[i]), t3(w1, 0), t3(y1[i]), t3(dw1, 0), 1,
+                                         t3(d2[i]), t3(x2[i]), t3(w2, 0), t3(y2[i]), t3(dw2, 0), 1, code, code, code, 1e-6,
+                                         wbuf.data_ptr(), ws.value, cbuf.data_ptr(), ct.value, st) == 0, lib.rgd_last_error()
+    n = B * (T1 * C1 + T2 * C2) * es
+    api = None
+    if with_api:
+        xa = x1[0].clone().requires_grad_(True)
+        if T2 == 0:
+            m = rgd.FusedRMSNorm(C1, device="cuda", dtype=dtype)
+            api = lambda: torch.autograd.grad(m(xa), (xa, m.weight), d1[0])
+        else:
+            xb = x2[0].clone().requires_grad_(True)
+            m = rgd.FusedRMSNorm2((C1, C2), device="cuda", dtype=dtype)
+            api = lambda: torch.autograd.grad(m(xa, xb), (xa, xb, m.weight1, m.weight2), (d1[0], d2[0]))
+    return rows_result(torch, name, fwd, bwd, 2 * n, 3 * n, nsets, api)
+
+
+def head_ln_case(torch, name, B, T, H, D, dtype, nsets):
+    import rgd_triton_amd as rgd
+    from rgd_triton_amd import _hip
+
+    lib = _hip.lib()
+    code = _hip.dtype_code(dtype)
+    st = _hip.stream_ptr(torch.device("cuda"))
+    mk = lambda: [torch.randn(B, T, H, D, device="cuda").to(dtype) for _ in range(nsets)]
+    q, k, gq, gk = mk(), mk(), mk(), mk()
+    qo, ko = [torch.empty_like(t) for t in q], [torch.empty_like(t) for t in k]
+    d = [{n: _hip.t4(x[i], False) for n, x in dict(q=q, k=k, gq=gq, gk=gk, qo=qo, ko=ko).items()} for i in range(nsets)]
+
+    def fwd(i):
+        assert lib.rgd_ln_qk_fwd(B, H, T, T, D, d[i]["q"], d[i]["k"], d[i]["qo"], d[i]["ko"], code, 1e-6, st) == 0, \
+            lib.rgd_last_error()
+
+    def bwd(i):
+        assert lib.rgd_ln_qk_bwd(B, H, T, T, D, d[i]["q"], d[i]["k"], d[i]["gq"], d[i]["gk"], d[i]["qo"], d[i]["ko"], code,
+                                 1e-6, st) == 0, lib.rgd_last_error()
+
+    qa, ka = q[0].clone().requires_grad_(True), k[0].clone().requires_grad_(True)
+    m = rgd.FusedHeadLayerNorm()
+    api = lambda: torch.autograd.grad(m(qa, ka, heads_second=False), (qa, ka), (gq[0], gk[0]))
+    n = 2 * B * T * H * D * torch.empty(0, dtype=dtype).element_size()
+    return rows_result(torch, name, fwd, bwd, 2 * n, 3 * n, nsets, api)
 
 
 def extras(torch, only=""):
@@ -243,29 +340,16 @@ def extras(torch, only=""):
     if want("attn_c5"):
         out.append(attention_case(torch, "attn_c5: (2,4352,24,64) bf16 broadcast bias", 2, 4352, 24, 64, bf, "broadcast"))
 
+    # buffer sets are sized so that their sum exceeds the 256 MB Infinity Cache
     if want("rms_c1"):
-        def mk_rms(i):
-            x = torch.randn(4, 1024, 1024, device="cuda", requires_grad=True)
-            m = rgd.FusedRMSNorm(1024, device="cuda")
-            dy = torch.randn_like(x)
-            return lambda: torch.autograd.grad(m(x), (x, m.weight), dy)
-        out.append(rows_case(torch, "rms_c1: FusedRMSNorm (4,1024,1024) fp32 fwd+bwd", mk_rms, 83886080, nsets=8))
+        out.append(rms_case(torch, "rms_c1: FusedRMSNorm (4,1024,1024) fp32 fwd+bwd", 4, [(1024, 1024)], torch.float32, 12))
     if want("rms2_c5"):
-        def mk_rms2(i):
-            x1 = torch.randn(2, 4096, 1536, device="cuda", dtype=bf, requires_grad=True)
-            x2 = torch.randn(2, 256, 1536, device="cuda", dtype=bf, requires_grad=True)
-            m = rgd.FusedRMSNorm2((1536, 1536), device="cuda", dtype=bf)
-            d1, d2 = torch.randn_like(x1), torch.randn_like(x2)
-            return lambda: torch.autograd.grad(m(x1, x2), (x1, x2, m.weight1, m.weight2), (d1, d2))
-        out.append(rows_case(torch, "rms2_c5: FusedRMSNorm2 (2,4096,1536)+(2,256,1536) bf16 fwd+bwd", mk_rms2, 133693440, nsets=6))
+        out.append(rms_case(torch, "rms2_c5: FusedRMSNorm2 (2,4096,1536)+(2,256,1536) bf16 fwd+bwd", 2,
+                            [(4096, 1536), (256, 1536)], bf, 12))
+    if want("rms_wide"):
+        out.append(rms_case(torch, "rms_wide: FusedRMSNorm (8,4096,4096) bf16 fwd+bwd", 8, [(4096, 4096)], bf, 3, with_api=False))
     if want("headln_c5"):
-        def mk_ln(i):
-            q = torch.randn(2, 4352, 24, 64, device="cuda", dtype=bf, requires_grad=True)
-            k = torch.randn(2, 4352, 24, 64, device="cuda", dtype=bf, requires_grad=True)
-            m = rgd.FusedHeadLayerNorm()
-            d1, d2 = torch.randn_like(q), torch.randn_like(k)
-            return lambda: torch.autograd.grad(m(q, k, heads_second=False), (q, k), (d1, d2))
-        out.append(rows_case(torch, "headln_c5: FusedHeadLayerNorm q,k (2,4352,24,64) bf16 fwd+bwd", mk_ln, 267386880, nsets=4))
+        out.append(head_ln_case(torch, "headln_c5: FusedHeadLayerNorm q,k (2,4352,24,64) bf16 fwd+bwd", 2, 4352, 24, 64, bf, 6))
     return out
 
 

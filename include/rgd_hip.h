@@ -72,11 +72,11 @@ int rgd_rms_fwd(int64_t B, int64_t T, int64_t C,
                 int x_dtype, int w_dtype, float eps, void* stream);
 
 /* Scratch the backward needs for the deterministic dw reduction.
- * *workspace_bytes: size of `workspace` (any contents on entry).
- * *counter_bytes:   size of `counters`; MUST be zero-filled before the first call that uses the
- *                   buffer; every call leaves it zero-filled again, so it can be reused by
- *                   successive calls on one stream without clearing.  Calls that may overlap
- *                   (different streams) need separate counter and workspace buffers. */
+ * *workspace_bytes: size of `workspace` (any contents on entry): one fp32 partial dw row per block, which
+ *                   a second small kernel adds in a fixed order.  Calls that may overlap (different
+ *                   streams) need separate workspaces.
+ * *counter_bytes:   always 0 in this version; the `counters` argument of the backward calls is kept in
+ *                   the interface and ignored (it may be null). */
 int rgd_rms_bwd_workspace(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2,
                           size_t* workspace_bytes, size_t* counter_bytes);
 

@@ -7,16 +7,19 @@
 // wavefront.  rrms / rlen are recomputed in the backward from x, which is being read anyway.
 //
 // dw of RMSNorm: every lane accumulates xhat*dy for its own channels over the rows of the block;
-// lanes, then waves, are combined in a fixed order into one fp32 partial row per block; partial rows
-// are combined by a fan-in-16 tree in which the last block to arrive at a node (atomic ticket) adds
-// the node's children in index order.  The result is independent of scheduling.
+// lanes, then waves, are combined in a fixed order into one fp32 partial row per block.  A second, small
+// kernel (wide_dw_reduce_kernel) adds the partial rows of a weight in a fixed order.  The result is
+// independent of scheduling.  (Combining the rows inside the first kernel, with arrival tickets, was
+// measured slower: every level of such a tree costs several microseconds of cross-XCD round trips.)
 #pragma once
 
 #include "common.h"
 
 enum { WIDE_RMS = 0, WIDE_L2 = 1 };
-constexpr int WIDE_FANIN = 16;
-constexpr int WIDE_MAX_LEVELS = 5;
+#ifndef RGD_WIDE_EPL_U2
+#define RGD_WIDE_EPL_U2 16  // backward: two rows in flight up to this many elements per lane
+#endif
+constexpr int WIDE_RED_WAVES = 8;  // wavefronts of a reduce block; each adds every 8th partial row
 
 struct WideHalf {
     const void* x;
@@ -28,12 +31,9 @@ struct WideHalf {
     int T, C, nchunks;
     int w_dtype, w_shared, w_vec;
     float inv_c;
-    float* part;  // partial rows of every tree level
-    int* ctr;     // arrival counters of every tree node (zero on entry, zero on exit)
-    int nleaf;    // leaves per tree
-    int tree_rows, tree_ctrs;
-    int lvl_row_off[WIDE_MAX_LEVELS];
-    int lvl_ctr_off[WIDE_MAX_LEVELS];
+    float* part;  // (weights, nleaf, C) partial rows, one per block
+    int nleaf;    // partial rows per weight
+    int red_blocks;  // reduce-kernel blocks of this half: weights * ceil(C / 64)
 };
 
 struct WideParams {
@@ -47,8 +47,7 @@ struct WideParams {
 // too wide to keep x, dy, w and the dw accumulators of one row in the registers of 64 lanes.
 template <typename T, int OP, bool BWD, int G, int NV, int VEC, bool VECTOR, int U, int NW, int WPR>
 __global__ __launch_bounds__(NW * 64) void wide_rows_kernel(const WideParams p) {
-    extern __shared__ float s_dw[];
-    __shared__ int s_last;
+    extern __shared__ __attribute__((aligned(16))) float s_dw[];  // backward with weights: NW/WPR rows of C sums
     __shared__ float s_red[2][2][NW];  // [parity][statistic][wavefront]
     static_assert(WPR == 1 || G == 64, "multi-wavefront rows use whole wavefronts");
 
@@ -178,79 +177,47 @@ __global__ __launch_bounds__(NW * 64) void wide_rows_kernel(const WideParams p) 
     }
 
     if constexpr (BWD && HAS_W) {
-        // ---- block partial: lanes that share channels, then waves, in a fixed order ----
+        // ---- block partial: lanes that share channels, then the wavefronts' rows, in a fixed order ----
 #pragma unroll
         for (int k = 0; k < NV; ++k)
 #pragma unroll
             for (int e = 0; e < VEC; ++e) dwacc[k][e] = cross_group_sum<G>(dwacc[k][e]);
-        // wavefront w covers the channels of row position (w % WPR); the first WPR wavefronts store, the
-        // others add, one wavefront at a time
-        for (int wv_i = 0; wv_i < NW; ++wv_i) {
-            if (wave == wv_i && lane < G) {
+        // every wavefront (every group of WPR wavefronts) leaves its sums in an LDS row of its own, all at
+        // once; then each thread adds the rows for a few channels in row order
+        constexpr int NR = NW / WPR;
+        float* my_row = s_dw + (wave / WPR) * C;
+        if (lane < G) {
 #pragma unroll
-                for (int k = 0; k < NV; ++k)
+            for (int k = 0; k < NV; ++k) {
+                const int c0 = (k * GL + lg) * VEC;
+                if (VECTOR && VEC % 4 == 0 && (C & 3) == 0) {  // C % 4 == 0: chunks are whole and 16-byte aligned
+                    if (c0 < C) {
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e) {
-                        const int c = (k * GL + lg) * VEC + e;
-                        if (c < C) s_dw[c] = wv_i < WPR ? dwacc[k][e] : s_dw[c] + dwacc[k][e];
+                        for (int e = 0; e < VEC; e += 4)
+                            *reinterpret_cast<f32x4*>(my_row + c0 + e) =
+                                f32x4{dwacc[k][e], dwacc[k][e + 1], dwacc[k][e + 2], dwacc[k][e + 3]};
                     }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e)
+                        if (c0 + e < C) my_row[c0 + e] = dwacc[k][e];
+                }
             }
-            if (wv_i % WPR == WPR - 1) __syncthreads();
         }
+        __syncthreads();
 
-        const int tree = h.w_shared ? 0 : b;
-        int idx = h.w_shared ? b * h.nchunks + chunk : chunk;
-        int n = h.nleaf;
-        void* dw_row = static_cast<char*>(h.dw) + (int64_t)tree * h.sdw_b * (h.w_dtype == RGD_F32 ? 4 : 2);
-        if (n == 1) {
-            for (int c = threadIdx.x; c < C; c += NW * 64) store_dyn(dw_row, h.w_dtype, c, s_dw[c]);
-            return;
-        }
-        float* tree_part = h.part + (int64_t)tree * h.tree_rows * C;
-        int* tree_ctr = h.ctr + (int64_t)tree * h.tree_ctrs;
-        // Partial rows travel between blocks through agent-scope (write-through) stores and loads, and
-        // each block waits for its own stores to complete before it takes a ticket.  That is all the
-        // ordering the tree needs, and it avoids a release fence, which on this multi-XCD part would
-        // write back the whole L2 (full of freshly written dx) once per block.
-        {
-            float* mine = tree_part + (int64_t)(h.lvl_row_off[0] + idx) * C;
-            for (int c = threadIdx.x; c < C; c += NW * 64)
-                __hip_atomic_store(mine + c, s_dw[c], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        for (int lvl = 0;; ++lvl) {
-            const int g = idx / WIDE_FANIN;
-            const int gs = min(WIDE_FANIN, n - g * WIDE_FANIN);
-            __builtin_amdgcn_s_waitcnt(0);  // this thread's partial-row stores have completed
-            __syncthreads();
-            if (threadIdx.x == 0) {
-                int* cp = tree_ctr + h.lvl_ctr_off[lvl] + g;
-                const int t = __hip_atomic_fetch_add(cp, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                const int last = (t == gs - 1);
-                if (last) __hip_atomic_store(cp, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                s_last = last;
-            }
-            __syncthreads();
-            if (!s_last) return;  // block-uniform
-            const int ng = (n + WIDE_FANIN - 1) / WIDE_FANIN;
-            const float* src = tree_part + (int64_t)(h.lvl_row_off[lvl] + g * WIDE_FANIN) * C;
-            float* dst = tree_part + (int64_t)(h.lvl_row_off[lvl + 1] + g) * C;
-            for (int c = threadIdx.x; c < C; c += NW * 64) {
-                float v[WIDE_FANIN];
+        const int wgt = h.w_shared ? 0 : b;  // which weight this block contributes to
+        const int idx = h.w_shared ? b * h.nchunks + chunk : chunk;
+        void* dw_row = static_cast<char*>(h.dw) + (int64_t)wgt * h.sdw_b * (h.w_dtype == RGD_F32 ? 4 : 2);
+        float* mine = h.part + ((int64_t)wgt * h.nleaf + idx) * C;
+        for (int c = threadIdx.x; c < C; c += NW * 64) {
+            float tot = s_dw[c];
 #pragma unroll
-                for (int j = 0; j < WIDE_FANIN; ++j)
-                    v[j] = j < gs ? __hip_atomic_load(src + (int64_t)j * C + c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-                                  : 0.f;
-                float acc = 0.f;
-#pragma unroll
-                for (int j = 0; j < WIDE_FANIN; ++j) acc += v[j];  // fixed order
-                if (ng == 1)
-                    store_dyn(dw_row, h.w_dtype, c, acc);
-                else
-                    __hip_atomic_store(dst + c, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-            if (ng == 1) return;
-            idx = g;
-            n = ng;
+            for (int r = 1; r < NR; ++r) tot += s_dw[r * C + c];
+            if (h.nleaf == 1)
+                store_dyn(dw_row, h.w_dtype, c, tot);
+            else
+                mine[c] = tot;
         }
     }
 }
@@ -280,6 +247,9 @@ struct WideConfig {
     bool vector;
 };
 // compile-time launch shape shared by the kernel instantiations and the host-side grid computation
-constexpr int wide_unroll(bool bwd, int nv) { return bwd ? (nv == 1 ? 2 : 1) : (nv == 1 ? 4 : (nv == 2 ? 2 : 1)); }
+// rows a lane group has in flight at once, by the elements of one row a lane holds (nv chunks of vec)
+constexpr int wide_unroll(bool bwd, int nv, int vec) {
+    return bwd ? (nv * vec <= RGD_WIDE_EPL_U2 ? 2 : 1) : (nv * vec <= 8 ? 4 : (nv * vec <= 16 ? 2 : 1));
+}
 constexpr int wide_waves(int op, bool bwd) { return (bwd && op == WIDE_RMS) ? 8 : 4; }
 template <typename T> int wide_dispatch(const WideConfig& cfg, const WideParams& p, dim3 grid, size_t lds, hipStream_t s);

@@ -7,9 +7,13 @@
 
 int rgd_num_cus();  // api.hip
 
+#ifndef RGD_DW_BLOCKS_PER_CU
+#define RGD_DW_BLOCKS_PER_CU 1
+#endif
+
 namespace {
 
-constexpr int DW_BLOCKS_PER_CU = 1;  // leaves of the dw tree per compute unit (RMSNorm backward)
+constexpr int DW_BLOCKS_PER_CU = RGD_DW_BLOCKS_PER_CU;  // blocks (= partial dw rows) per compute unit, RMSNorm backward
 constexpr int BLOCKS_PER_CU = 8;     // target grid size of the other kernels
 
 int pow2ceil(int v) {
@@ -18,35 +22,45 @@ int pow2ceil(int v) {
     return p;
 }
 
-struct TreeShape {
-    int rows = 0, ctrs = 0;
-    int row_off[WIDE_MAX_LEVELS] = {0}, ctr_off[WIDE_MAX_LEVELS] = {0};
-};
-
-TreeShape tree_shape(int nleaf) {
-    TreeShape t;
-    int n = nleaf, lvl = 0;
-    while (n > 1 && lvl < WIDE_MAX_LEVELS) {
-        t.row_off[lvl] = t.rows;
-        t.ctr_off[lvl] = t.ctrs;
-        t.rows += n;
-        n = (n + WIDE_FANIN - 1) / WIDE_FANIN;
-        t.ctrs += n;
-        ++lvl;
-    }
-    if (lvl < WIDE_MAX_LEVELS) t.row_off[lvl] = t.rows;
-    return t;
+// upper bound of the partial rows one half can need, whatever tile shape is chosen later
+size_t half_bound(int64_t B, int64_t T, int64_t target) {
+    return T <= 0 ? 0 : (size_t)target + (size_t)B + 8;
 }
 
-// upper bound of partial rows / counters one half can need, whatever tile shape is chosen later
-void half_bound(int64_t B, int64_t T, int64_t target, size_t* rows, size_t* ctrs) {
-    if (T <= 0) {
-        *rows = *ctrs = 0;
-        return;
+// dw[weight][c] = sum over the partial rows of that weight, in a fixed order: wavefront w of the block adds
+// rows w, w+8, w+16, ... for 64 consecutive channels, then the 8 wavefront sums are added in index order.
+__global__ __launch_bounds__(WIDE_RED_WAVES * 64) void wide_dw_reduce_kernel(const WideParams p) {
+    __shared__ float s_sum[WIDE_RED_WAVES][64];
+    const int which = (int)blockIdx.x >= p.h[0].red_blocks ? 1 : 0;
+    const WideHalf& h = p.h[which];
+    const int blk = blockIdx.x - (which ? p.h[0].red_blocks : 0);
+    const int cblocks = (h.C + 63) / 64;
+    const int wgt = blk / cblocks;
+    const int lane = lane_id(), wave = threadIdx.x >> 6;
+    const int c = (blk - wgt * cblocks) * 64 + lane;
+    const float* src = h.part + (int64_t)wgt * h.nleaf * h.C + c;
+    float acc = 0.f;
+    if (c < h.C) {
+        int r = wave;
+#pragma unroll 1
+        for (; r + 3 * WIDE_RED_WAVES < h.nleaf; r += 4 * WIDE_RED_WAVES) {  // four loads in flight
+            const float v0 = src[(int64_t)r * h.C];
+            const float v1 = src[(int64_t)(r + WIDE_RED_WAVES) * h.C];
+            const float v2 = src[(int64_t)(r + 2 * WIDE_RED_WAVES) * h.C];
+            const float v3 = src[(int64_t)(r + 3 * WIDE_RED_WAVES) * h.C];
+            acc = (((acc + v0) + v1) + v2) + v3;
+        }
+        for (; r < h.nleaf; r += WIDE_RED_WAVES) acc += src[(int64_t)r * h.C];
     }
-    const size_t leaves = (size_t)target + (size_t)B;
-    *rows = leaves + leaves / 8 + 8 * (size_t)B + 8;
-    *ctrs = leaves / 8 + 8 * (size_t)B + 8;
+    s_sum[wave][lane] = acc;
+    __syncthreads();
+    if (wave == 0 && c < h.C) {
+        float tot = s_sum[0][lane];
+#pragma unroll
+        for (int w = 1; w < WIDE_RED_WAVES; ++w) tot += s_sum[w][lane];
+        void* dw_row = static_cast<char*>(h.dw) + (int64_t)wgt * h.sdw_b * (h.w_dtype == RGD_F32 ? 4 : 2);
+        store_dyn(dw_row, h.w_dtype, c, tot);
+    }
 }
 
 bool t3_vec_ok(const rgd_tensor3* t, int es) {
@@ -57,17 +71,17 @@ bool t3_vec_ok(const rgd_tensor3* t, int es) {
 
 int wide_workspace(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2, size_t* ws, size_t* ctr) {
     const int64_t target = (int64_t)rgd_num_cus() * DW_BLOCKS_PER_CU;
-    size_t r1, c1, r2, c2;
-    half_bound(B, T1, target, &r1, &c1);
-    half_bound(B, T2, target, &r2, &c2);
+    const size_t r1 = half_bound(B, T1, target), r2 = half_bound(B, T2, target);
     *ws = (r1 * (size_t)std::max<int64_t>(C1, 0) + r2 * (size_t)std::max<int64_t>(C2, 0)) * sizeof(float);
-    *ctr = (c1 + c2) * sizeof(int);
+    *ctr = 0;  // no counters are needed; the argument stays in the interface
     return RGD_OK;
 }
 
 int wide_launch(const char* name, int op, bool bwd, int64_t B, const WideHalfArgs& a1, const WideHalfArgs& a2,
                 int dtype, float eps, void* workspace, size_t workspace_bytes, void* counters,
                 size_t counter_bytes, void* stream) {
+    (void)counters;  // kept in the interface, not used
+    (void)counter_bytes;
     RGD_REQUIRE(rgd_dtype_ok(dtype), RGD_ERR_INVALID, "%s: Only support fp16, bf16, and fp32", name);
     RGD_REQUIRE(B >= 0 && B <= 65535, RGD_ERR_INVALID, "%s: batch %lld out of range", name, (long long)B);
     const WideHalfArgs* as[2] = {&a1, &a2};
@@ -126,7 +140,7 @@ int wide_launch(const char* name, int op, bool bwd, int64_t B, const WideHalfArg
                     256 * max_epl);
     }
     const int NW = wide_waves(op, bwd);
-    const int U = wide_unroll(bwd, cfg.NV);
+    const int U = wide_unroll(bwd, cfg.NV, vec);
     const int row_quantum = NW * (64 / cfg.G) / cfg.WPR * U;
     const bool tree = has_w && bwd;
     const int64_t target = (int64_t)rgd_num_cus() * (tree ? DW_BLOCKS_PER_CU : BLOCKS_PER_CU);
@@ -138,8 +152,8 @@ int wide_launch(const char* name, int op, bool bwd, int64_t B, const WideHalfArg
     memset(&p, 0, sizeof(p));
     p.rows_per_chunk = (int)rpc;
     p.eps = eps;
-    size_t ws_used = 0, ctr_used = 0;
-    int64_t grid_x = 0;
+    size_t ws_used = 0;
+    int64_t grid_x = 0, red_grid = 0;
     for (int i = 0; i < 2; ++i) {
         const WideHalfArgs* a = as[i];
         WideHalf& h = p.h[i];
@@ -176,31 +190,24 @@ int wide_launch(const char* name, int op, bool bwd, int64_t B, const WideHalfArg
             h.sdw_b = a->dw->stride_b;
             h.w_shared = a->w_shared ? 1 : 0;
             h.nleaf = h.w_shared ? (int)B * h.nchunks : h.nchunks;
-            const int ntrees = h.w_shared ? 1 : (int)B;
-            const TreeShape ts = tree_shape(h.nleaf);
-            h.tree_rows = ts.rows;
-            h.tree_ctrs = ts.ctrs;
-            for (int l = 0; l < WIDE_MAX_LEVELS; ++l) {
-                h.lvl_row_off[l] = ts.row_off[l];
-                h.lvl_ctr_off[l] = ts.ctr_off[l];
-            }
+            const int nweights = h.w_shared ? 1 : (int)B;
             h.part = reinterpret_cast<float*>(static_cast<char*>(workspace) + ws_used);
-            h.ctr = reinterpret_cast<int*>(static_cast<char*>(counters) + ctr_used);
-            ws_used += (size_t)ntrees * ts.rows * a->C * sizeof(float);
-            ctr_used += (size_t)ntrees * ts.ctrs * sizeof(int);
+            if (h.nleaf > 1) {
+                ws_used += (size_t)nweights * h.nleaf * a->C * sizeof(float);
+                h.red_blocks = nweights * (int)((a->C + 63) / 64);
+                red_grid += h.red_blocks;
+            }
         }
     }
     if (tree) {
-        RGD_REQUIRE(ws_used <= workspace_bytes && ctr_used <= counter_bytes, RGD_ERR_WORKSPACE,
-                    "%s: workspace too small (need %zu + %zu bytes, have %zu + %zu)", name, ws_used, ctr_used,
-                    workspace_bytes, counter_bytes);
-        RGD_REQUIRE((ws_used == 0 || workspace) && (ctr_used == 0 || counters), RGD_ERR_INVALID,
-                    "%s: null workspace", name);
+        RGD_REQUIRE(ws_used <= workspace_bytes, RGD_ERR_WORKSPACE, "%s: workspace too small (need %zu bytes, have %zu)",
+                    name, ws_used, workspace_bytes);
+        RGD_REQUIRE(ws_used == 0 || workspace, RGD_ERR_INVALID, "%s: null workspace", name);
     }
     RGD_REQUIRE(grid_x < (1ll << 31), RGD_ERR_UNSUPPORTED, "%s: grid too large", name);
 
     const dim3 grid((unsigned)grid_x, (unsigned)B, 1);
-    const size_t lds = tree ? (size_t)maxC * sizeof(float) : 0;
+    const size_t lds = tree ? (size_t)(NW / cfg.WPR) * maxC * sizeof(float) : 0;  // one row of sums per wavefront group
     RGD_REQUIRE(lds <= 64 * 1024, RGD_ERR_UNSUPPORTED, "%s: row too wide for the dw staging buffer", name);
     hipStream_t s = static_cast<hipStream_t>(stream);
     int rc;
@@ -212,6 +219,10 @@ int wide_launch(const char* name, int op, bool bwd, int64_t B, const WideHalfArg
         rc = wide_dispatch<bf16_t>(cfg, p, grid, lds, s);
     if (rc != RGD_OK) return rc;
     RGD_CHECK_LAUNCH(name);
+    if (red_grid > 0) {  // dw = fixed-order sum of the blocks' partial rows
+        hipLaunchKernelGGL(wide_dw_reduce_kernel, dim3((unsigned)red_grid), dim3(WIDE_RED_WAVES * 64), 0, s, p);
+        RGD_CHECK_LAUNCH(name);
+    }
     return RGD_OK;
 }
 

@@ -8,7 +8,7 @@
 template <typename T, int OP, bool BWD, int G, int NV, bool VECTOR, int WPR>
 static int wide_launch_one(const WideParams& p, dim3 grid, size_t lds, hipStream_t s) {
     constexpr int VEC = VECTOR ? 16 / (int)sizeof(T) : 2;
-    constexpr int U = wide_unroll(BWD, NV);
+    constexpr int U = wide_unroll(BWD, NV, VEC);
     constexpr int NW = wide_waves(OP, BWD);
     // the host never selects more elements per lane than this (they would not stay in registers)
     if constexpr (NV * VEC <= (OP == WIDE_RMS ? 32 : 64)) {

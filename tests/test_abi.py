@@ -61,7 +61,8 @@ def test_error_paths_return_codes_without_a_gpu():
     assert lib.rgd_l2_fwd(0, 0, 8, t3, t3, 0, 1e-6, None) == 0
     ws, ct = ctypes.c_size_t(), ctypes.c_size_t()
     assert lib.rgd_rms_bwd_workspace(4, 1024, 1024, 0, 0, ctypes.byref(ws), ctypes.byref(ct)) == 0
-    assert ws.value >= 256 * 1024 * 4 and ct.value >= 16 * 4
+    # one fp32 partial dw row per block; no counters are used (the argument stays in the interface)
+    assert ws.value >= 256 * 1024 * 4 and ct.value == 0
     # a too small workspace is refused before any launch
     assert lib.rgd_rms_bwd(4, 1024, 1024, t3, t3, t3, t3, t3, 1, 0, 0, 1e-6, 0x1000, 16, 0x1000, 4, None) == -4
 
