@@ -189,6 +189,7 @@ def attention_case(torch, name, B, T, H, D, dtype, bias_kind, iters=20):
     tqr = lib.rgd_attn_seqlen_q_rounded(T)
     lse = torch.empty(B, H, tqr, dtype=torch.float32, device="cuda")
     ws = torch.empty(lib.rgd_attn_bwd_workspace(B, H, T, T, D), dtype=torch.uint8, device="cuda")
+    fws = torch.empty(max(lib.rgd_attn_fwd_workspace(B, H, T, T, D), 16), dtype=torch.uint8, device="cuda")
     code = _hip.dtype_code(dtype)
     if bias is None:
         bdesc, bk, bd = _hip.Tensor4(None, 0, 0, 0), _hip.BIAS_NONE, _hip.RGD_F32
@@ -201,7 +202,7 @@ def attention_case(torch, name, B, T, H, D, dtype, bias_kind, iters=20):
 
     def fwd():
         assert lib.rgd_attn_fwd(B, H, T, T, D, t["q"], t["k"], t["v"], bdesc, bk, bd, t["o"], lse.data_ptr(), code, 0,
-                                scale, st) == 0, lib.rgd_last_error()
+                                scale, fws.data_ptr(), fws.numel(), st) == 0, lib.rgd_last_error()
 
     def bwd():
         assert lib.rgd_attn_bwd(B, H, T, T, D, t["do"], t["q"], t["k"], t["v"], t["o"], lse.data_ptr(), bdesc, bk, bd,

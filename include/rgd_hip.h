@@ -201,9 +201,19 @@ int rgd_attn_fwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D,
                  const rgd_tensor4* q, const rgd_tensor4* k, const rgd_tensor4* v,
                  const rgd_tensor4* bias, int bias_kind, int bias_dtype,
                  const rgd_tensor4* o, float* lse,
-                 int dtype, int causal, float softmax_scale, void* stream);
+                 int dtype, int causal, float softmax_scale,
+                 void* workspace, size_t workspace_bytes, void* stream);
 
-/* bytes of scratch rgd_attn_bwd needs (delta, fp32 (B,H,Tq_rounded)); any contents on entry */
+/* Optional scratch of rgd_attn_fwd (any contents on entry, 16-byte aligned).  With it, the query blocks of
+ * the last, partly filled round of workgroups are split along the keys and merged by a second launch, which
+ * fills the chip for grids that are not a multiple of the resident workgroups (and for small grids).
+ * workspace = NULL or a smaller buffer is legal: the call then splits less or not at all.  Results do not
+ * depend on scheduling; a split item sums its keys in a different grouping than an unsplit one. */
+size_t rgd_attn_fwd_workspace(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D);
+
+/* bytes of scratch for rgd_attn_bwd (any contents on entry, 16-byte aligned): delta, fp32 (B,H,Tq_rounded),
+ * which is required, then room for the fp32 partial sums of split workgroups (as in rgd_attn_fwd_workspace),
+ * which is optional: a workspace that only holds delta is accepted and nothing is split. */
 size_t rgd_attn_bwd_workspace(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D);
 
 /* replaces _flash_attn_backward, flash_attn/flash_attn_triton_cached.py:885-1075

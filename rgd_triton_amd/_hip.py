@@ -55,7 +55,8 @@ _SIGNATURES = {
     "rgd_ln_rope_qk_bwd": (_int, [_i64] * 5 + [_T4] * 6 + [_vp, _i64, _i64, _i64, _i64, _int, _i64, _i64, _int, _f32,
                                                             _vp]),
     "rgd_attn_seqlen_q_rounded": (_i64, [_i64]),
-    "rgd_attn_fwd": (_int, [_i64] * 5 + [_T4] * 4 + [_int, _int, _T4, _vp, _int, _int, _f32, _vp]),
+    "rgd_attn_fwd": (_int, [_i64] * 5 + [_T4] * 4 + [_int, _int, _T4, _vp, _int, _int, _f32, _vp, _sz, _vp]),
+    "rgd_attn_fwd_workspace": (_sz, [_i64] * 5),
     "rgd_attn_bwd_workspace": (_sz, [_i64] * 5),
     "rgd_attn_bwd": (_int, [_i64] * 5 + [_T4] * 5 + [_vp] + [_T4, _int, _int] + [_T4] * 3 + [_int, _int, _f32, _vp, _sz,
                                                                                          _vp]),

@@ -8,6 +8,9 @@
 
 // kernel instantiations live in attn_f16.hip / attn_bf16.hip (attn_inst.h) so they compile in parallel
 template <typename T> int dispatch_fwd(const AttnFwdParams& p, unsigned grid, hipStream_t s);
+template <typename T> int dispatch_fwd_merge(const AttnFwdParams& p, unsigned items, hipStream_t s);
+template <typename T> int dispatch_bwd_merge(const AttnBwdParams& p, unsigned items, int nt, hipStream_t s);
+int rgd_num_cus();  // api.hip
 template <typename T, bool DQ> int dispatch_bwd(const AttnBwdParams& p, unsigned grid, hipStream_t s);
 
 namespace {
@@ -23,6 +26,17 @@ AttnTensor at(const rgd_tensor4* t) {
     a.sn = t ? t->stride_n : 0;
     return a;
 }
+
+int attn_dpad(int64_t D) { return D <= 32 ? 32 : D <= 64 ? 64 : D <= 96 ? 96 : 128; }
+// resident workgroups per compute unit of the forward kernel (its launch bounds and LDS use)
+int fwd_blocks_per_cu(int dpad, bool bias) { return (dpad <= 64 && !bias) ? 3 : 2; }
+// bytes one part of a split forward item leaves behind: 128 rows of accumulators, exponent and row sum
+size_t fwd_part_bytes(int dpad) { return (size_t)ATTN_BM * dpad * sizeof(float) + (size_t)ATTN_BM * 2 * sizeof(float); }
+
+// resident workgroups per compute unit of the backward kernels, and the bytes a part of a split item leaves
+int bwd_blocks_per_cu(int dpad) { return dpad <= 64 ? 2 : 1; }
+size_t bwd_part_bytes(int dpad, int tensors) { return (size_t)tensors * BWD_BM * dpad * sizeof(float); }
+size_t bwd_delta_bytes(int64_t B, int64_t H, int64_t Tq) { return (size_t)(B * H * rgd_attn_seqlen_q_rounded(Tq)) * sizeof(float); }
 
 int check_common(const char* name, int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, int dtype, int bias_kind,
                  int bias_dtype, const rgd_tensor4* bias) {
@@ -51,9 +65,15 @@ extern "C" {
 
 int64_t rgd_attn_seqlen_q_rounded(int64_t Tq) { return (Tq + 63) / 64 * 64; }
 
+size_t rgd_attn_fwd_workspace(int64_t, int64_t, int64_t, int64_t, int64_t D) {
+    if (D < 1 || D > 128) return 0;
+    return (size_t)2 * rgd_num_cus() * 3 * fwd_part_bytes(attn_dpad(D));  // two rounds of parts at the highest occupancy
+}
+
 int rgd_attn_fwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const rgd_tensor4* q, const rgd_tensor4* k,
                  const rgd_tensor4* v, const rgd_tensor4* bias, int bias_kind, int bias_dtype, const rgd_tensor4* o,
-                 float* lse, int dtype, int causal, float softmax_scale, void* stream) {
+                 float* lse, int dtype, int causal, float softmax_scale, void* workspace, size_t workspace_bytes,
+                 void* stream) {
     const char* name = "rgd_attn_fwd";
     int rc = check_common(name, B, H, Tq, Tk, D, dtype, bias_kind, bias_dtype, bias);
     if (rc != RGD_OK) return rc;
@@ -91,17 +111,39 @@ int rgd_attn_fwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
         p.bias_vec = rgd_aligned16(bias->ptr) && (p.bias.sb % per16) == 0 && (p.bias.sh % per16) == 0 &&
                      (p.bias.sn % per16) == 0;
     }
-    const int64_t grid = (int64_t)p.nqb * B * H;
+    const int64_t items = (int64_t)p.nqb * B * H;
+    // items of the last, partly filled round are split along the keys when a workspace is given
+    const int dpad = attn_dpad(D);
+    AttnSplit plan;
+    if (workspace && rgd_aligned16(workspace) && !causal)
+        plan = attn_split_plan(items, rgd_num_cus() * fwd_blocks_per_cu(dpad, bias_kind != RGD_BIAS_NONE),
+                               (int)((Tk + ATTN_BN - 1) / ATTN_BN), fwd_part_bytes(dpad), workspace_bytes);
+    p.split_full = plan.full;
+    p.split_s = plan.s;
+    if (plan.s > 1) {
+        const size_t parts = (size_t)plan.items_split(items) * plan.s;
+        p.part_o = static_cast<float*>(workspace);
+        p.part_ml = p.part_o + parts * ATTN_BM * dpad;
+    }
+    const int64_t grid = plan.blocks(items);
     RGD_REQUIRE(grid < (1ll << 31), RGD_ERR_UNSUPPORTED, "%s: grid too large", name);
     hipStream_t s = static_cast<hipStream_t>(stream);
     rc = dtype == RGD_F16 ? dispatch_fwd<f16_t>(p, (unsigned)grid, s) : dispatch_fwd<bf16_t>(p, (unsigned)grid, s);
     if (rc != RGD_OK) return rc;
     RGD_CHECK_LAUNCH(name);
+    if (plan.s > 1) {
+        const unsigned n = (unsigned)plan.items_split(items);
+        rc = dtype == RGD_F16 ? dispatch_fwd_merge<f16_t>(p, n, s) : dispatch_fwd_merge<bf16_t>(p, n, s);
+        if (rc != RGD_OK) return rc;
+        RGD_CHECK_LAUNCH(name);
+    }
     return RGD_OK;
 }
 
-size_t rgd_attn_bwd_workspace(int64_t B, int64_t H, int64_t Tq, int64_t, int64_t) {
-    return (size_t)(B * H * rgd_attn_seqlen_q_rounded(Tq)) * sizeof(float);
+size_t rgd_attn_bwd_workspace(int64_t B, int64_t H, int64_t Tq, int64_t, int64_t D) {
+    // delta, then room for two rounds of dK/dV parts (the dQ parts reuse it; the launches are ordered)
+    const int dpad = attn_dpad(D < 1 ? 1 : D);
+    return bwd_delta_bytes(B, H, Tq) + (size_t)2 * rgd_num_cus() * bwd_blocks_per_cu(dpad) * bwd_part_bytes(dpad, 2);
 }
 
 int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const rgd_tensor4* dout, const rgd_tensor4* q,
@@ -117,8 +159,15 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
     for (const rgd_tensor4* t : all) RGD_REQUIRE(t, RGD_ERR_INVALID, "%s: null tensor descriptor", name);
     RGD_REQUIRE(Tq == 0 || (dout->ptr && q->ptr && o->ptr && dq->ptr && lse), RGD_ERR_INVALID, "%s: null tensor", name);
     RGD_REQUIRE(Tk == 0 || (k->ptr && v->ptr && dk->ptr && dv->ptr), RGD_ERR_INVALID, "%s: null tensor", name);
-    RGD_REQUIRE(workspace_bytes >= rgd_attn_bwd_workspace(B, H, Tq, Tk, D) && (workspace || Tq == 0), RGD_ERR_WORKSPACE,
-                "%s: workspace too small", name);
+    // delta is required; whatever the workspace holds beyond it is used to split the last round of workgroups
+    const size_t delta_bytes = bwd_delta_bytes(B, H, Tq);
+    RGD_REQUIRE(workspace_bytes >= delta_bytes && (workspace || Tq == 0), RGD_ERR_WORKSPACE, "%s: workspace too small",
+                name);
+    const int dpad = attn_dpad(D);
+    const bool may_split = workspace && rgd_aligned16(workspace) && !causal;
+    float* part_base = reinterpret_cast<float*>(static_cast<char*>(workspace) + delta_bytes);
+    const size_t part_room = workspace_bytes - delta_bytes;
+    const int slots = rgd_num_cus() * bwd_blocks_per_cu(dpad);
 
     AttnBwdParams p;
     memset(&p, 0, sizeof(p));
@@ -155,19 +204,43 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (Tq > 0) {  // dQ and delta
         p.nblk = (int)((Tq + BWD_BM - 1) / BWD_BM);
-        const int64_t grid = (int64_t)p.nblk * B * H;
+        const int64_t items = (int64_t)p.nblk * B * H;
+        AttnSplit plan;
+        if (may_split) plan = attn_split_plan(items, slots, (int)((Tk + 63) / 64), bwd_part_bytes(dpad, 1), part_room);
+        p.split_full = plan.full;
+        p.split_s = plan.s;
+        p.part = part_base;
+        const int64_t grid = plan.blocks(items);
         RGD_REQUIRE(grid < (1ll << 31), RGD_ERR_UNSUPPORTED, "%s: grid too large", name);
         rc = dtype == RGD_F16 ? dispatch_bwd<f16_t, true>(p, (unsigned)grid, s) : dispatch_bwd<bf16_t, true>(p, (unsigned)grid, s);
         if (rc != RGD_OK) return rc;
         RGD_CHECK_LAUNCH(name);
+        if (plan.s > 1) {
+            const unsigned n = (unsigned)plan.items_split(items);
+            rc = dtype == RGD_F16 ? dispatch_bwd_merge<f16_t>(p, n, 1, s) : dispatch_bwd_merge<bf16_t>(p, n, 1, s);
+            if (rc != RGD_OK) return rc;
+            RGD_CHECK_LAUNCH(name);
+        }
     }
     if (Tk > 0) {  // dK and dV (reads delta)
         p.nblk = (int)((Tk + BWD_BM - 1) / BWD_BM);
-        const int64_t grid = (int64_t)p.nblk * B * H;
+        const int64_t items = (int64_t)p.nblk * B * H;
+        AttnSplit plan;
+        if (may_split) plan = attn_split_plan(items, slots, (int)((Tq + 63) / 64), bwd_part_bytes(dpad, 2), part_room);
+        p.split_full = plan.full;
+        p.split_s = plan.s;
+        p.part = part_base;
+        const int64_t grid = plan.blocks(items);
         RGD_REQUIRE(grid < (1ll << 31), RGD_ERR_UNSUPPORTED, "%s: grid too large", name);
         rc = dtype == RGD_F16 ? dispatch_bwd<f16_t, false>(p, (unsigned)grid, s) : dispatch_bwd<bf16_t, false>(p, (unsigned)grid, s);
         if (rc != RGD_OK) return rc;
         RGD_CHECK_LAUNCH(name);
+        if (plan.s > 1) {
+            const unsigned n = (unsigned)plan.items_split(items);
+            rc = dtype == RGD_F16 ? dispatch_bwd_merge<f16_t>(p, n, 2, s) : dispatch_bwd_merge<bf16_t>(p, n, 2, s);
+            if (rc != RGD_OK) return rc;
+            RGD_CHECK_LAUNCH(name);
+        }
     }
     return RGD_OK;
 }

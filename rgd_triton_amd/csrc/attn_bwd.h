@@ -31,7 +31,37 @@ struct AttnBwdParams {
     int B, H, Tq, Tk, D, Tq_rounded, nblk;
     int bias_kind, bias_dtype, bias_vec, causal, vec;
     float scale, scale_log2;
+    // split of the last round of workgroups (AttnSplit), set separately for the dQ and the dK/dV launch:
+    // hardware blocks >= split_full are part (id % split_s) of item split_full + id / split_s and leave fp32
+    // partial sums in `part`, (parts, 128, DPAD) for dQ and (parts, 2, 128, DPAD) for dK, dV
+    int split_full, split_s;
+    float* part;
 };
+
+// block id -> (logical item, part, number of parts, part id)
+struct BwdItem {
+    int bid, part, nparts, part_id;
+};
+__device__ __forceinline__ BwdItem bwd_item(const AttnBwdParams& p) {
+    BwdItem it{0, 0, 1, 0};
+    if (p.split_s <= 1) {
+        it.bid = xcd_remap(blockIdx.x, gridDim.x);
+    } else if ((int)blockIdx.x < p.split_full) {
+        it.bid = xcd_remap(blockIdx.x, p.split_full);
+    } else {
+        it.part_id = blockIdx.x - p.split_full;
+        it.bid = p.split_full + it.part_id / p.split_s;
+        it.part = it.part_id % p.split_s;
+        it.nparts = p.split_s;
+    }
+    return it;
+}
+
+// 16 contiguous columns of one row of an fp32 partial tile
+__device__ __forceinline__ void store_part16(float* row, int col, const f32x16& acc) {
+#pragma unroll
+    for (int e = 0; e < 16; e += 4) *reinterpret_cast<f32x4*>(row + col + e) = f32x4{acc[e], acc[e + 1], acc[e + 2], acc[e + 3]};
+}
 
 template <int DPAD> struct BwdTile {
     static constexpr int S = attn_lds_stride(DPAD);  // row stride of every staged tile (elements)
@@ -90,7 +120,8 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dq_k
     T* const vs_base = ks_base + 2 * TILE;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 31, g = lane >> 5;
-    const int bid = xcd_remap(blockIdx.x, gridDim.x);
+    const BwdItem item = bwd_item(p);
+    const int bid = item.bid;
     const int qb = bid % p.nblk;
     const int bh = bid / p.nblk;
     const int b = bh / p.H, h = bh - b * p.H;
@@ -119,7 +150,7 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dq_k
     const float lse = p.lse[(int64_t)bh * p.Tq_rounded + min(q_row, p.Tq_rounded - 1)];
     // rows that do not exist, and rows whose logits are all -inf, get probability 0 everywhere
     const float neg_lse_l2 = (q_valid && lse != -INFINITY) ? -lse * kLog2e : -INFINITY;
-    if (g == 0 && q_row < p.Tq_rounded) p.delta[(int64_t)bh * p.Tq_rounded + q_row] = q_valid ? delta : 0.f;
+    if (g == 0 && q_row < p.Tq_rounded && item.part == 0) p.delta[(int64_t)bh * p.Tq_rounded + q_row] = q_valid ? delta : 0.f;
     f32x16 dp_init;  // -delta in every element: what the dP accumulators start from
 #pragma unroll
     for (int v = 0; v < 16; ++v) dp_init[v] = -delta;
@@ -132,6 +163,9 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dq_k
 
     int ntiles = (p.Tk + BN - 1) / BN;
     if (p.causal) ntiles = min(ntiles, (min(p.Tq, (qb + 1) * BWD_BM) + BN - 1) / BN);
+    // this workgroup's share of the key tiles (all of them unless the item is split)
+    const int t_begin = (int)((int64_t)ntiles * item.part / item.nparts);
+    const int t_end = (int)((int64_t)ntiles * (item.part + 1) / item.nparts);
 
     const T* kbase = static_cast<const T*>(p.k.ptr) + b * p.k.sb + h * p.k.sh;
     const T* vbase = static_cast<const T*>(p.v.ptr) + b * p.v.sb + h * p.v.sh;
@@ -173,9 +207,9 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dq_k
             *reinterpret_cast<u32x4*>(vs_base + buf * TILE + soff[i]) = vst[i];
         }
     };
-    if (ntiles > 0) {
-        issue_loads(0);
-        store_tiles(0);
+    if (t_begin < t_end) {
+        issue_loads(t_begin);
+        store_tiles(t_begin & 1);
     }
     __syncthreads();
 
@@ -185,14 +219,14 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dq_k
     BiasRuns<TB> bias_cur, bias_nxt;  // fetched one tile ahead of use
     if constexpr (HAS_BIAS) {
         bias_row = static_cast<const TB*>(p.bias.ptr) + b * p.bias.sb + h * p.bias.sh + (int64_t)q_ld * p.bias.sn;
-        if (ntiles > 0) bias_cur.load(bias_row, 0, g, p.Tk, p.bias_vec && BN <= p.Tk);
+        if (t_begin < t_end) bias_cur.load(bias_row, t_begin * BN, g, p.Tk, p.bias_vec && (t_begin + 1) * BN <= p.Tk);
     }
 
-    for (int j = 0; j < ntiles; ++j) {
+    for (int j = t_begin; j < t_end; ++j) {
         const int buf = j & 1;
         const int key0 = j * BN;
         const bool tail = key0 + BN > p.Tk;
-        if (j + 1 < ntiles) {
+        if (j + 1 < t_end) {
             issue_loads(j + 1);
             if constexpr (HAS_BIAS) bias_nxt.load(bias_row, key0 + BN, g, p.Tk, p.bias_vec && key0 + 2 * BN <= p.Tk);
         }
@@ -268,13 +302,19 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dq_k
                 acc[d] = MM::run(as_v8<T>(a), bop, acc[d]);
             }
         }
-        if (j + 1 < ntiles) {
+        if (j + 1 < t_end) {
             store_tiles(buf ^ 1);
             if constexpr (HAS_BIAS) bias_cur = bias_nxt;
         }
         __syncthreads();
     }
 
+    if (item.nparts > 1) {  // part of a split item: leave the unscaled fp32 sums
+        float* row = p.part + ((int64_t)item.part_id * BWD_BM + wave * 32 + li) * DPAD;
+#pragma unroll
+        for (int d = 0; d < NDB; ++d) store_part16(row, d * 32 + g * 16, acc[d]);
+        return;
+    }
     if (q_valid) {
         T* dqp = static_cast<T*>(const_cast<void*>(p.dq.ptr)) + b * p.dq.sb + h * p.dq.sh + (int64_t)q_row * p.dq.sn;
 #pragma unroll
@@ -348,7 +388,8 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_D
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 31, g = lane >> 5;
-    const int bid = xcd_remap(blockIdx.x, gridDim.x);
+    const BwdItem item = bwd_item(p);
+    const int bid = item.bid;
     const int kblk = bid % p.nblk;
     const int bh = bid / p.nblk;
     const int b = bh / p.H, h = bh - b * p.H;
@@ -379,8 +420,11 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_D
             dv_acc[d][v] = 0.f;
         }
 
-    const int ntiles = (p.Tq + BQ - 1) / BQ;
-    const int tile_begin = p.causal ? min(ntiles, (kblk * BWD_BM) / BQ) : 0;
+    // this workgroup's share of the query tiles (all of them unless the item is split)
+    const int ntiles_all = (p.Tq + BQ - 1) / BQ;
+    const int tile_first = p.causal ? min(ntiles_all, (kblk * BWD_BM) / BQ) : 0;
+    const int tile_begin = tile_first + (int)((int64_t)(ntiles_all - tile_first) * item.part / item.nparts);
+    const int ntiles = tile_first + (int)((int64_t)(ntiles_all - tile_first) * (item.part + 1) / item.nparts);
 
     int ld_row[LOADS], ld_dc[LOADS], qoff[LOADS], dooff[LOADS], soff[LOADS];
 #pragma unroll
@@ -567,6 +611,15 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_D
         __syncthreads();
     }
 
+    if (item.nparts > 1) {  // part of a split item: leave the unscaled fp32 sums, dK then dV
+        float* row = p.part + (((int64_t)item.part_id * 2) * BWD_BM + wave * 32 + li) * DPAD;
+#pragma unroll
+        for (int d = 0; d < NDB; ++d) {
+            store_part16(row, d * 32 + g * 16, dk_acc[d]);
+            store_part16(row + (int64_t)BWD_BM * DPAD, d * 32 + g * 16, dv_acc[d]);
+        }
+        return;
+    }
     if (k_valid) {
         T* dkp = static_cast<T*>(const_cast<void*>(p.dk.ptr)) + b * p.dk.sb + h * p.dk.sh + (int64_t)key * p.dk.sn;
         T* dvp = static_cast<T*>(const_cast<void*>(p.dv.ptr)) + b * p.dv.sb + h * p.dv.sh + (int64_t)key * p.dv.sn;
@@ -575,5 +628,38 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_D
             store_row16<T>(dkp, d * 32 + g * 16, p.D, vec, dk_acc[d], p.scale);
             store_row16<T>(dvp, d * 32 + g * 16, p.D, vec, dv_acc[d], 1.0f);
         }
+    }
+}
+
+// Adds the fp32 partial tiles of split items in part order and writes the rows in the tensor dtype.
+// NT = tensors per item (1: dQ, 2: dK and dV).  One thread per (row, 4 consecutive columns);
+// grid (split items, ceil(128 * DPAD/4 / 256), NT).
+template <typename T, int DPAD> __global__ __launch_bounds__(256) void attn_bwd_merge_kernel(const AttnBwdParams p, int nt) {
+    constexpr int CPR = DPAD / 4;
+    const int id = blockIdx.y * 256 + threadIdx.x;
+    if (id >= BWD_BM * CPR) return;
+    const int row = id / CPR, col = (id - row * CPR) * 4;
+    const int which = blockIdx.z;
+    const int item = p.split_full + blockIdx.x;
+    const int blk = item % p.nblk, bh = item / p.nblk;
+    const int b = bh / p.H, h = bh - b * p.H;
+    const int t_row = blk * BWD_BM + row;
+    const AttnTensor& out = nt == 1 ? p.dq : (which == 0 ? p.dk : p.dv);
+    const int limit = nt == 1 ? p.Tq : p.Tk;
+    const float mul = (nt == 2 && which == 1) ? 1.0f : p.scale;
+    if (t_row >= limit) return;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < p.split_s; ++i) {
+        const float* src = p.part + ((((int64_t)blockIdx.x * p.split_s + i) * nt + which) * BWD_BM + row) * DPAD + col;
+        acc += *reinterpret_cast<const f32x4*>(src);
+    }
+    T* op = static_cast<T*>(const_cast<void*>(out.ptr)) + b * out.sb + h * out.sh + (int64_t)t_row * out.sn;
+    if (p.vec && col + 4 <= p.D) {
+        const uint32_t w0 = pack2<T>(acc[0] * mul, acc[1] * mul), w1 = pack2<T>(acc[2] * mul, acc[3] * mul);
+        *reinterpret_cast<u32x2*>(op + col) = u32x2{w0, w1};
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (col + e < p.D) op[col + e] = static_cast<T>(acc[e] * mul);
     }
 }

@@ -175,5 +175,37 @@ struct AttnTensor {
     int64_t sb, sh, sn;
 };
 
+// A launch of `items` equal workgroups on `slots` resident workgroup slots runs in ceil(items/slots) rounds and
+// the last round may be nearly empty.  The plan keeps the first `full` items (whole rounds) as they are and
+// splits each of the remaining items into `s` parts along its inner loop, so the last round is 1/s as long;
+// a merge kernel combines the parts.  s == 1: no split.  Host side only.
+struct AttnSplit {
+    int full = 0, s = 1;
+    int items_split(int64_t items) const { return s > 1 ? (int)(items - full) : 0; }
+    int64_t blocks(int64_t items) const { return s > 1 ? full + (items - full) * s : items; }
+};
+inline AttnSplit attn_split_plan(int64_t items, int slots, int inner_tiles, size_t part_bytes, size_t workspace_bytes) {
+    AttnSplit plan;
+    if (items <= 0 || slots <= 0 || items >= (1ll << 30)) return plan;
+    const int64_t full = items / slots * slots, rest = items - full;
+    if (rest == 0) return plan;
+    double best = 1.0;
+    for (int s = 2; s <= 8; ++s) {
+        if (inner_tiles < 2 * s) break;                                   // parts of at least two tiles
+        if (rest * s > 2 * (int64_t)slots) break;                         // at most two rounds of parts
+        if ((size_t)(rest * s) * part_bytes > workspace_bytes) break;     // what the caller's workspace holds
+        const double cost = (double)((rest * s + slots - 1) / slots) / s;  // length of the split round
+        if (cost < best - 1e-9) {
+            best = cost;
+            plan.s = s;
+        }
+    }
+    // worth the partial results and a merge launch only if the last round shrinks to half or less and that
+    // saves the equivalent of a dozen tile steps
+    if (plan.s > 1 && (best > 0.5 || (1.0 - best) * inner_tiles < 12.0)) plan.s = 1;
+    plan.full = plan.s > 1 ? (int)full : 0;
+    return plan;
+}
+
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;

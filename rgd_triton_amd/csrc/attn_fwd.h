@@ -34,6 +34,12 @@ struct AttnFwdParams {
     int B, H, Tq, Tk, D, Tq_rounded, nqb;
     int bias_kind, bias_dtype, bias_vec, causal, vec;
     float scale_log2;  // softmax_scale * log2(e)
+    // Split of the last, partly filled round of workgroups (see AttnSplit): hardware blocks below split_full
+    // are whole items; the others are part (id % split_s) of item split_full + id / split_s and leave
+    // unnormalised partial results, which attn_fwd_merge_kernel combines.  split_s <= 1: no split.
+    int split_full, split_s;
+    float* part_o;   // (parts, 128, DPAD) fp32 accumulators, relative to the part's reference exponent
+    float* part_ml;  // (parts, 128, 2): reference exponent (log2 domain), sum of probabilities
 };
 
 template <int DPAD> struct AttnFwdSmem {
@@ -68,7 +74,17 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
     const int li = lane & 31;
     const int g = lane >> 5;
 
-    const int bid = xcd_remap(blockIdx.x, gridDim.x);
+    int bid, part = 0, nparts = 1, part_id = 0;
+    if (p.split_s <= 1) {
+        bid = xcd_remap(blockIdx.x, gridDim.x);
+    } else if ((int)blockIdx.x < p.split_full) {
+        bid = xcd_remap(blockIdx.x, p.split_full);
+    } else {
+        part_id = blockIdx.x - p.split_full;
+        bid = p.split_full + part_id / p.split_s;
+        part = part_id % p.split_s;
+        nparts = p.split_s;
+    }
     const int qb = bid % p.nqb;
     const int bh = bid / p.nqb;
     const int b = bh / p.H;
@@ -95,6 +111,8 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
 
     int ntiles = (p.Tk + ATTN_BN - 1) / ATTN_BN;
     if (p.causal) ntiles = min(ntiles, (min(p.Tq, (qb + 1) * ATTN_BM) + ATTN_BN - 1) / ATTN_BN);
+    // this workgroup's share of the key tiles (all of them unless the item is split)
+    const int t_begin = (int)((int64_t)ntiles * part / nparts), t_end = (int)((int64_t)ntiles * (part + 1) / nparts);
 
     // global -> register staging of the next tile.  Thread t moves the 16-byte chunks t, t+256, ... of the
     // tile; its offsets inside a tile are fixed, the tile base is wavefront-uniform.
@@ -144,9 +162,9 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
         }
     };
 
-    if (ntiles > 0) {
-        issue_loads(0);
-        store_tiles(0);
+    if (t_begin < t_end) {
+        issue_loads(t_begin);
+        store_tiles(t_begin & 1);
     }
     __syncthreads();
 
@@ -160,14 +178,15 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
     BiasRuns<TB> bias_cur, bias_nxt;
     if constexpr (HAS_BIAS) {
         bias_row = static_cast<const TB*>(p.bias.ptr) + b * p.bias.sb + h * p.bias.sh + (int64_t)q_ld * p.bias.sn;
-        if (ntiles > 0) bias_cur.load(bias_row, 0, g, p.Tk, p.bias_vec && ATTN_BN <= p.Tk);
+        if (t_begin < t_end)
+            bias_cur.load(bias_row, t_begin * ATTN_BN, g, p.Tk, p.bias_vec && (t_begin + 1) * ATTN_BN <= p.Tk);
     }
 
-    for (int j = 0; j < ntiles; ++j) {
+    for (int j = t_begin; j < t_end; ++j) {
         const int buf = j & 1;
         const int key0 = j * ATTN_BN;
         const bool tail = key0 + ATTN_BN > p.Tk;
-        if (j + 1 < ntiles) {
+        if (j + 1 < t_end) {
             issue_loads(j + 1);
             if constexpr (HAS_BIAS)
                 bias_nxt.load(bias_row, key0 + ATTN_BN, g, p.Tk, p.bias_vec && key0 + 2 * ATTN_BN <= p.Tk);
@@ -357,15 +376,32 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
             }
         }
 
-        if (j + 1 < ntiles) {
+        if (j + 1 < t_end) {
             store_tiles(buf ^ 1);
             if constexpr (HAS_BIAS) bias_cur = bias_nxt;
         }
         __syncthreads();
     }
 
-    // ---- epilogue: normalise, write O and LSE ----
     const float l_tot = l_run + lane_xor32(l_run);
+    if (nparts > 1) {
+        // ---- part of a split item: leave the unnormalised accumulators, m_ref and the row sum ----
+        const int row = wave * 32 + li;
+        float* po = p.part_o + ((int64_t)part_id * ATTN_BM + row) * DPAD;
+#pragma unroll
+        for (int d = 0; d < NDB; ++d)
+#pragma unroll
+            for (int e = 0; e < 16; e += 4)
+                *reinterpret_cast<f32x4*>(po + d * 32 + g * 16 + e) =
+                    f32x4{oacc[d][e], oacc[d][e + 1], oacc[d][e + 2], oacc[d][e + 3]};
+        if (g == 0) {
+            float* pm = p.part_ml + ((int64_t)part_id * ATTN_BM + row) * 2;
+            pm[0] = m_ref;
+            pm[1] = l_tot;
+        }
+        return;
+    }
+    // ---- epilogue: normalise, write O and LSE ----
     const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
     T* op = static_cast<T*>(const_cast<void*>(p.o.ptr)) + b * p.o.sb + h * p.o.sh + (int64_t)q_row * p.o.sn;
     if (q_valid) {
@@ -395,4 +431,43 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
         const float lse = q_valid ? (m_ref + __builtin_amdgcn_logf(l_tot)) * kLn2 : 0.f;
         p.lse[(int64_t)bh * p.Tq_rounded + q_row] = lse;
     }
+}
+
+// Combines the parts of split items: for every row, m = max m_i, O = sum_i 2^(m_i - m) O_i / sum_i 2^(m_i - m) l_i,
+// in part order.  One thread per (row, 4 consecutive columns); grid (split items, ceil(128 * DPAD/4 / 256)).
+template <typename T, int DPAD> __global__ __launch_bounds__(256) void attn_fwd_merge_kernel(const AttnFwdParams p) {
+    constexpr int CPR = DPAD / 4;  // 4-column chunks per row
+    const int id = blockIdx.y * 256 + threadIdx.x;
+    if (id >= ATTN_BM * CPR) return;
+    const int row = id / CPR, col = (id - row * CPR) * 4;
+    const int item = p.split_full + blockIdx.x;
+    const int qb = item % p.nqb, bh = item / p.nqb;
+    const int b = bh / p.H, h = bh - b * p.H;
+    const int q_row = qb * ATTN_BM + row;
+    const int64_t part0 = (int64_t)blockIdx.x * p.split_s;
+    float m = -INFINITY;
+    for (int i = 0; i < p.split_s; ++i) m = fmaxf(m, p.part_ml[((part0 + i) * ATTN_BM + row) * 2]);
+    float l = 0.f;
+    f32x4 o = {0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < p.split_s; ++i) {
+        const float* pm = p.part_ml + ((part0 + i) * ATTN_BM + row) * 2;
+        const float w = pm[0] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(pm[0] - m);
+        l += w * pm[1];
+        const f32x4 oi = *reinterpret_cast<const f32x4*>(p.part_o + ((part0 + i) * ATTN_BM + row) * DPAD + col);
+        o += oi * w;
+    }
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    if (q_row < p.Tq) {
+        T* op = static_cast<T*>(const_cast<void*>(p.o.ptr)) + b * p.o.sb + h * p.o.sh + (int64_t)q_row * p.o.sn;
+        if (p.vec && col + 4 <= p.D) {
+            const uint32_t w0 = pack2<T>(o[0] * inv, o[1] * inv), w1 = pack2<T>(o[2] * inv, o[3] * inv);
+            *reinterpret_cast<u32x2*>(op + col) = u32x2{w0, w1};
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (col + e < p.D) op[col + e] = static_cast<T>(o[e] * inv);
+        }
+    }
+    if (col == 0 && q_row < p.Tq_rounded)
+        p.lse[(int64_t)bh * p.Tq_rounded + q_row] = q_row < p.Tq ? (m + __builtin_amdgcn_logf(l)) * kLn2 : 0.f;
 }

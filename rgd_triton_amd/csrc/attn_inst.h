@@ -21,6 +21,19 @@ template <typename T, int DPAD, int BIAS> int launch_fwd(const AttnFwdParams& p,
     return RGD_OK;
 }
 
+template <typename T, int DPAD> int launch_fwd_merge(const AttnFwdParams& p, unsigned items, hipStream_t s) {
+    const unsigned gy = (ATTN_BM * (DPAD / 4) + 255) / 256;
+    hipLaunchKernelGGL((attn_fwd_merge_kernel<T, DPAD>), dim3(items, gy), dim3(256), 0, s, p);
+    return RGD_OK;
+}
+
+template <typename T> int dispatch_fwd_merge(const AttnFwdParams& p, unsigned items, hipStream_t s) {
+    if (p.D <= 32) return launch_fwd_merge<T, 32>(p, items, s);
+    if (p.D <= 64) return launch_fwd_merge<T, 64>(p, items, s);
+    if (p.D <= 96) return launch_fwd_merge<T, 96>(p, items, s);
+    return launch_fwd_merge<T, 128>(p, items, s);
+}
+
 template <typename T> int dispatch_fwd(const AttnFwdParams& p, unsigned grid, hipStream_t s) {
     const int bias = p.bias_kind == RGD_BIAS_NONE ? BIAS_OFF : (p.bias_dtype == RGD_F32 ? BIAS_F32 : BIAS_SAME);
 #define FWD_CASE(DP)                                                                 \
@@ -67,3 +80,16 @@ template <typename T, bool DQ> int dispatch_bwd(const AttnBwdParams& p, unsigned
     return RGD_ERR_UNSUPPORTED;
 }
 
+
+template <typename T, int DPAD> int launch_bwd_merge(const AttnBwdParams& p, unsigned items, int nt, hipStream_t s) {
+    const unsigned gy = (BWD_BM * (DPAD / 4) + 255) / 256;
+    hipLaunchKernelGGL((attn_bwd_merge_kernel<T, DPAD>), dim3(items, gy, nt), dim3(256), 0, s, p, nt);
+    return RGD_OK;
+}
+
+template <typename T> int dispatch_bwd_merge(const AttnBwdParams& p, unsigned items, int nt, hipStream_t s) {
+    if (p.D <= 32) return launch_bwd_merge<T, 32>(p, items, nt, s);
+    if (p.D <= 64) return launch_bwd_merge<T, 64>(p, items, nt, s);
+    if (p.D <= 96) return launch_bwd_merge<T, 96>(p, items, nt, s);
+    return launch_bwd_merge<T, 128>(p, items, nt, s);
+}

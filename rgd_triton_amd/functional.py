@@ -493,10 +493,11 @@ def _flash_attn_forward(q, k, v, bias=None, causal=False, softmax_scale=None, ke
     seqlen_q_rounded = lib.rgd_attn_seqlen_q_rounded(seqlen_q)
     lse = torch.empty((batch, nheads, seqlen_q_rounded), device=q.device, dtype=torch.float32)
     o = torch.empty_like(q)
+    ws = _hip.scratch(q.device, "attn_fwd_ws", lib.rgd_attn_fwd_workspace(batch, nheads, seqlen_q, seqlen_k, d))
     _hip.check(lib.rgd_attn_fwd(batch, nheads, seqlen_q, seqlen_k, d, t4(q, False), t4(k, False), t4(v, False),
                                 bdesc, bkind, bdtype, t4(o, False), ctypes.c_void_p(lse.data_ptr()),
                                 _hip.dtype_code(q.dtype), int(bool(causal)), float(softmax_scale),
-                                _hip.stream_ptr(q.device)), "rgd_attn_fwd")
+                                ctypes.c_void_p(ws.data_ptr()), ws.numel(), _hip.stream_ptr(q.device)), "rgd_attn_fwd")
     return o, lse, softmax_scale
 
 

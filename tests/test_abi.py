@@ -25,7 +25,8 @@ def test_library_exports_every_declared_symbol():
     assert lib.rgd_version() == 1000
     assert lib.rgd_attn_seqlen_q_rounded(1) == 64 and lib.rgd_attn_seqlen_q_rounded(128) == 128
     assert lib.rgd_attn_seqlen_q_rounded(129) == 192
-    assert lib.rgd_attn_bwd_workspace(2, 3, 100, 50, 64) == 2 * 3 * 128 * 4
+    # delta (required part) plus room for the partial sums of split workgroups
+    assert lib.rgd_attn_bwd_workspace(2, 3, 100, 50, 64) >= 2 * 3 * 128 * 4
 
 
 def test_header_cites_the_reference_for_every_entry_point():
@@ -50,11 +51,11 @@ def test_error_paths_return_codes_without_a_gpu():
     assert lib.rgd_rope_qk(1, 1, 4, 4, 160, t4, t4, t4, t4, 0x1000, 8, 32, 256, 32, 0, 4, 4, 0, 0, None) == -1
     assert b"head dimensions up to 128" in lib.rgd_last_error()
     assert lib.rgd_rope_qk(1, 1, 8, 8, 64, t4, t4, t4, t4, 0x1000, 8, 32, 256, 32, 0, 8, 8, 0, 0, None) == -1  # T < P
-    assert lib.rgd_attn_fwd(1, 1, 8, 8, 64, t4, t4, t4, None, 0, 0, t4, 0x1000, 0, 0, 0.125, None) == -1
+    assert lib.rgd_attn_fwd(1, 1, 8, 8, 64, t4, t4, t4, None, 0, 0, t4, 0x1000, 0, 0, 0.125, None, 0, None) == -1
     assert b"Only support fp16 and bf16" in lib.rgd_last_error()
-    assert lib.rgd_attn_fwd(1, 1, 8, 8, 200, t4, t4, t4, None, 0, 0, t4, 0x1000, 1, 0, 0.125, None) == -1
+    assert lib.rgd_attn_fwd(1, 1, 8, 8, 200, t4, t4, t4, None, 0, 0, t4, 0x1000, 1, 0, 0.125, None, 0, None) == -1
     assert b"head dimensions up to 128" in lib.rgd_last_error()
-    assert lib.rgd_attn_fwd(1, 1, 8, 8, 64, t4, t4, t4, t4, 2, 2, t4, 0x1000, 1, 0, 0.125, None) == -1  # bias dtype
+    assert lib.rgd_attn_fwd(1, 1, 8, 8, 64, t4, t4, t4, t4, 2, 2, t4, 0x1000, 1, 0, 0.125, None, 0, None) == -1  # bias dtype
     assert lib.rgd_attn_bwd(1, 1, 8, 8, 64, t4, t4, t4, t4, t4, 0x1000, None, 0, 0, t4, t4, t4, 1, 0, 0.125, 0x1000, 16,
                             None) == -4
     # zero-sized problems are a successful no-op
