@@ -266,3 +266,64 @@ def test_flash_attn_module_errors_and_cache():
     out = flash_attn_func(q, q, q, bias)
     with pytest.raises(AssertionError, match="does not support bias gradient"):
         out.sum().backward()
+
+
+@pytest.mark.parametrize("dtype", HALF)
+@pytest.mark.parametrize("B,H,T,d,with_bias", [(1, 2, 2048, 64, False), (1, 3, 1536, 128, True), (2, 5, 1100, 32, True)])
+def test_flash_attn_split_workgroups(B, H, T, d, with_bias, dtype):
+    """With a workspace the library splits the workgroups of a partly filled last round (here: a grid far
+    smaller than the chip) along their inner loop and merges fp32 partial results.  Through the C ABI: the
+    split run must agree with the unsplit run (no workspace / a workspace that only holds delta) to fp32
+    regrouping accuracy, must be bit-reproducible, and both must pass the oracle check."""
+    import ctypes
+    from rgd_triton_amd import _hip
+
+    lib = _hip.lib()
+    g = gen(11)
+    q, k, v, do = (randn(g, B, T, H, d, dtype=dtype) for _ in range(4))
+    bias = make_bias(g, "batch", B, H, T, T, dtype) if with_bias else None
+    qg, kg, vg, dog = (t.cuda() for t in (q, k, v, do))
+    code = _hip.dtype_code(dtype)
+    if bias is None:
+        bdesc, bk, bd = _hip.Tensor4(None, 0, 0, 0), _hip.BIAS_NONE, _hip.RGD_F32
+    else:
+        bg = bias.cuda()
+        be = bg.expand(B, H, T, T)
+        bdesc, bk, bd = _hip.Tensor4(be.data_ptr(), be.stride(0), be.stride(1), be.stride(2)), _hip.BIAS_MATRIX, code
+    st = _hip.stream_ptr(qg.device)
+    scale = 1.0 / math.sqrt(d)
+    tqr = lib.rgd_attn_seqlen_q_rounded(T)
+    delta_bytes = B * H * tqr * 4
+    full_f, full_b = lib.rgd_attn_fwd_workspace(B, H, T, T, d), lib.rgd_attn_bwd_workspace(B, H, T, T, d)
+    assert full_b > delta_bytes
+
+    def run(fws_bytes, bws_bytes):
+        o, dq, dk, dv = (torch.empty_like(qg) for _ in range(4))
+        lse = torch.empty(B, H, tqr, dtype=torch.float32, device="cuda")
+        fws = torch.empty(max(fws_bytes, 16), dtype=torch.uint8, device="cuda")
+        bws = torch.empty(bws_bytes, dtype=torch.uint8, device="cuda")
+        t = {n: _hip.t4(x, False) for n, x in dict(q=qg, k=kg, v=vg, do=dog, o=o, dq=dq, dk=dk, dv=dv).items()}
+        rc = lib.rgd_attn_fwd(B, H, T, T, d, t["q"], t["k"], t["v"], bdesc, bk, bd, t["o"], lse.data_ptr(), code, 0, scale,
+                              fws.data_ptr() if fws_bytes else None, fws_bytes, st)
+        assert rc == 0, lib.rgd_last_error()
+        rc = lib.rgd_attn_bwd(B, H, T, T, d, t["do"], t["q"], t["k"], t["v"], t["o"], lse.data_ptr(), bdesc, bk, bd, t["dq"],
+                              t["dk"], t["dv"], code, 0, scale, bws.data_ptr(), bws_bytes, st)
+        assert rc == 0, lib.rgd_last_error()
+        torch.cuda.synchronize()
+        return o, lse, dq, dk, dv
+
+    plain = run(0, delta_bytes)
+    split = run(full_f, full_b)
+    again = run(full_f, full_b)
+    for a, b_, n in zip(split, again, ("o", "lse", "dq", "dk", "dv")):
+        assert torch.equal(a, b_), f"{n}: the split run is not reproducible"
+    # same math, other summation grouping: agreement far inside one rounding step of the output type
+    ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+    for a, b_, n in zip(split, plain, ("o", "lse", "dq", "dk", "dv")):
+        scale_n = b_.float().abs().max().item()
+        assert maxdiff(a, b_.cpu()) <= (1e-5 if n == "lse" else 1.01 * ulp) * max(scale_n, 1.0), n
+    # the split really happened: regrouped fp32 sums differ in the last bit of some of the thousands of LSE rows
+    assert not torch.equal(split[1], plain[1])
+    ref = reference(q, k, v, bias, do)
+    check(split, ref, T, grad_mult=3, name="split")
+    check(plain, ref, T, grad_mult=3, name="unsplit")
