@@ -38,6 +38,11 @@ int bwd_blocks_per_cu(int dpad) { return dpad <= 64 ? 2 : 1; }
 size_t bwd_part_bytes(int dpad, int tensors) { return (size_t)tensors * BWD_BM * dpad * sizeof(float); }
 size_t bwd_delta_bytes(int64_t B, int64_t H, int64_t Tq) { return (size_t)(B * H * rgd_attn_seqlen_q_rounded(Tq)) * sizeof(float); }
 
+// measured: what a second and third resident workgroup add to a compute unit, and the duration of one inner
+// step (64 keys or 64 query rows) of a workgroup that has its compute unit to itself
+constexpr AttnSplitModel kFwdSplit = {1.3f, 1.5f, 0.9f};
+constexpr AttnSplitModel kBwdSplit = {1.05f, 1.05f, 1.4f};
+
 int check_common(const char* name, int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, int dtype, int bias_kind,
                  int bias_dtype, const rgd_tensor4* bias) {
     RGD_REQUIRE(dtype == RGD_F16 || dtype == RGD_BF16, RGD_ERR_INVALID, "%s: Only support fp16 and bf16", name);
@@ -116,8 +121,8 @@ int rgd_attn_fwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
     const int dpad = attn_dpad(D);
     AttnSplit plan;
     if (workspace && rgd_aligned16(workspace) && !causal)
-        plan = attn_split_plan(items, rgd_num_cus() * fwd_blocks_per_cu(dpad, bias_kind != RGD_BIAS_NONE),
-                               (int)((Tk + ATTN_BN - 1) / ATTN_BN), fwd_part_bytes(dpad), workspace_bytes);
+        plan = attn_split_plan(items, rgd_num_cus(), fwd_blocks_per_cu(dpad, bias_kind != RGD_BIAS_NONE),
+                               (int)((Tk + ATTN_BN - 1) / ATTN_BN), fwd_part_bytes(dpad), workspace_bytes, kFwdSplit);
     p.split_full = plan.full;
     p.split_s = plan.s;
     if (plan.s > 1) {
@@ -167,7 +172,7 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
     const bool may_split = workspace && rgd_aligned16(workspace) && !causal;
     float* part_base = reinterpret_cast<float*>(static_cast<char*>(workspace) + delta_bytes);
     const size_t part_room = workspace_bytes - delta_bytes;
-    const int slots = rgd_num_cus() * bwd_blocks_per_cu(dpad);
+    const int per_cu = bwd_blocks_per_cu(dpad);
 
     AttnBwdParams p;
     memset(&p, 0, sizeof(p));
@@ -206,7 +211,9 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
         p.nblk = (int)((Tq + BWD_BM - 1) / BWD_BM);
         const int64_t items = (int64_t)p.nblk * B * H;
         AttnSplit plan;
-        if (may_split) plan = attn_split_plan(items, slots, (int)((Tk + 63) / 64), bwd_part_bytes(dpad, 1), part_room);
+        if (may_split)
+            plan = attn_split_plan(items, rgd_num_cus(), per_cu, (int)((Tk + 63) / 64), bwd_part_bytes(dpad, 1), part_room,
+                                   kBwdSplit);
         p.split_full = plan.full;
         p.split_s = plan.s;
         p.part = part_base;
@@ -226,7 +233,9 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
         p.nblk = (int)((Tk + BWD_BM - 1) / BWD_BM);
         const int64_t items = (int64_t)p.nblk * B * H;
         AttnSplit plan;
-        if (may_split) plan = attn_split_plan(items, slots, (int)((Tq + 63) / 64), bwd_part_bytes(dpad, 2), part_room);
+        if (may_split)
+            plan = attn_split_plan(items, rgd_num_cus(), per_cu, (int)((Tq + 63) / 64), bwd_part_bytes(dpad, 2), part_room,
+                                   kBwdSplit);
         p.split_full = plan.full;
         p.split_s = plan.s;
         p.part = part_base;

@@ -175,34 +175,50 @@ struct AttnTensor {
     int64_t sb, sh, sn;
 };
 
-// A launch of `items` equal workgroups on `slots` resident workgroup slots runs in ceil(items/slots) rounds and
-// the last round may be nearly empty.  The plan keeps the first `full` items (whole rounds) as they are and
-// splits each of the remaining items into `s` parts along its inner loop, so the last round is 1/s as long;
-// a merge kernel combines the parts.  s == 1: no split.  Host side only.
+// A launch of `items` equal workgroups runs in rounds of cus * per_cu resident workgroups and the last round
+// may leave most of the chip idle.  The plan keeps the items of the whole rounds as they are and splits each
+// item of the last round into `s` parts along its inner loop; a merge kernel combines the parts' partial
+// results.  s == 1: no split.  Host side only.
+//
+// Cost model (measured on MI355X): a compute unit with n resident workgroups of these kernels delivers
+// thr(n) times the throughput of one workgroup alone, far below n (MFMA and VALU work of the wavefronts of a
+// SIMD add up); the last round's time is the work of its busiest compute unit divided by that throughput.
+// A split is taken when the time it saves exceeds the cost of writing, re-reading and merging the parts.
 struct AttnSplit {
     int full = 0, s = 1;
     int items_split(int64_t items) const { return s > 1 ? (int)(items - full) : 0; }
     int64_t blocks(int64_t items) const { return s > 1 ? full + (items - full) * s : items; }
 };
-inline AttnSplit attn_split_plan(int64_t items, int slots, int inner_tiles, size_t part_bytes, size_t workspace_bytes) {
+struct AttnSplitModel {
+    float thr2, thr3;  // throughput of a compute unit with 2 / 3 resident workgroups, relative to 1
+    float tile_us;     // one inner-loop step of a workgroup alone on its compute unit
+};
+inline AttnSplit attn_split_plan(int64_t items, int cus, int per_cu, int inner_tiles, size_t part_bytes,
+                                 size_t workspace_bytes, AttnSplitModel m) {
     AttnSplit plan;
-    if (items <= 0 || slots <= 0 || items >= (1ll << 30)) return plan;
+    if (items <= 0 || cus <= 0 || per_cu <= 0 || items >= (1ll << 30)) return plan;
+    const int64_t slots = (int64_t)cus * per_cu;
     const int64_t full = items / slots * slots, rest = items - full;
     if (rest == 0) return plan;
-    double best = 1.0;
+    auto round_time = [&](int64_t parts, int s) {  // in units of one whole item alone on a compute unit
+        const int64_t n = (parts + cus - 1) / cus;  // parts the busiest compute unit works through
+        const int64_t res = n < per_cu ? n : per_cu;
+        const double thr = res >= 3 ? m.thr3 : (res == 2 ? m.thr2 : 1.0);
+        return (double)n / thr / s;
+    };
+    const double item_us = (double)inner_tiles * m.tile_us, t1 = round_time(rest, 1);
+    double best_gain = 3.0;  // microseconds a split must save to be taken
     for (int s = 2; s <= 8; ++s) {
-        if (inner_tiles < 2 * s) break;                                   // parts of at least two tiles
-        if (rest * s > 2 * (int64_t)slots) break;                         // at most two rounds of parts
-        if ((size_t)(rest * s) * part_bytes > workspace_bytes) break;     // what the caller's workspace holds
-        const double cost = (double)((rest * s + slots - 1) / slots) / s;  // length of the split round
-        if (cost < best - 1e-9) {
-            best = cost;
+        if (inner_tiles < 2 * s) break;                                 // parts of at least two steps
+        if (rest * s > 2 * slots) break;                                // at most two rounds of parts
+        if ((size_t)(rest * s) * part_bytes > workspace_bytes) break;   // what the caller's workspace holds
+        const double overhead_us = 6.0 + (double)(rest * s) * part_bytes * 2.0 / 4.0e6;  // merge launch + traffic at 4 TB/s
+        const double gain = (t1 - round_time(rest * s, s)) * item_us - overhead_us;
+        if (gain > best_gain) {
+            best_gain = gain;
             plan.s = s;
         }
     }
-    // worth the partial results and a merge launch only if the last round shrinks to half or less and that
-    // saves the equivalent of a dozen tile steps
-    if (plan.s > 1 && (best > 0.5 || (1.0 - best) * inner_tiles < 12.0)) plan.s = 1;
     plan.full = plan.s > 1 ? (int)full : 0;
     return plan;
 }
