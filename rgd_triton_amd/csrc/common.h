@@ -106,11 +106,7 @@ __device__ __forceinline__ void store_chunk(T* __restrict__ p, int first, int li
                 for (int e = 0; e < EPV; ++e) tmp[e] = from_f32<T>(in[v * EPV + e]);
                 u32x4 raw;
                 __builtin_memcpy(&raw, tmp, 16);
-#if defined(RGD_NT_STORE)
-                __builtin_nontemporal_store(raw, vp + v);
-#else
                 vp[v] = raw;
-#endif
             }
         }
     } else {
@@ -124,7 +120,10 @@ __device__ __forceinline__ void store_chunk(T* __restrict__ p, int first, int li
 // range reads the start of the row instead, which is always valid memory) and out-of-range elements are
 // zeroed by a select when the raw bits are decoded.  Issue every load() of an iteration first, then
 // decode(): the loads overlap and the wavefront waits once.
-template <typename T, int N, bool VECTOR> struct Chunk {
+// NT: non-temporal loads (data that is read once and not shared between workgroups).  Measured: they
+// shorten forward kernels (one input stream) by 7-12 % and lengthen backward kernels (two input streams) by
+// 15 %.
+template <typename T, int N, bool VECTOR, bool NT = false> struct Chunk {
     static constexpr bool VEC = VECTOR && (N * sizeof(T)) % 16 == 0;
     static constexpr int NVEC = VEC ? (N * sizeof(T)) / 16 : 1;
     static constexpr int EPV = 16 / sizeof(T);
@@ -136,11 +135,10 @@ template <typename T, int N, bool VECTOR> struct Chunk {
             const u32x4* p = reinterpret_cast<const u32x4*>(row + (first < limit ? first : 0));
 #pragma unroll
             for (int i = 0; i < NVEC; ++i) {
-#if defined(RGD_NT_LOAD)
-                v[i] = __builtin_nontemporal_load(p + i);
-#else
-                v[i] = p[i];
-#endif
+                if constexpr (NT)
+                    v[i] = __builtin_nontemporal_load(p + i);
+                else
+                    v[i] = p[i];
             }
         } else {
 #pragma unroll

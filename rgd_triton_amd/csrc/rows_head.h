@@ -58,6 +58,8 @@ __global__ __launch_bounds__(256) void head_rows_kernel(const HeadParams p) {
     const uint32_t row0 = (blockIdx.x - (which ? p.blocks_q : 0u)) * (uint32_t)(ROWS_PER_PASS * U) + wave * GPW + lane / G;
     const int D = p.D;
 
+    // plain (temporal) loads on purpose: non-temporal loads of x shorten the forward by 7 % but leave nothing
+    // of q, k in the Infinity Cache for a backward that follows soon, which then takes 17 % longer
     Chunk<T, VEC, VECTOR> xc[U][NV], dc[U][NV];
     Chunk<TP, VEC, VECTOR> sc[U][NV], cc[U][NV];
     bool rotate[U];

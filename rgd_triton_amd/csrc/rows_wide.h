@@ -93,7 +93,8 @@ __global__ __launch_bounds__(NW * 64) void wide_rows_kernel(const WideParams p) 
     const int iters = (r1 - r0 + NSLOT * U - 1) / (NSLOT * U);
     for (int it = 0; it < iters; ++it) {
         const int rbase = r0 + slot + it * NSLOT * U;
-        Chunk<T, VEC, VECTOR> xc[U][NV], dc[U][NV];
+        Chunk<T, VEC, VECTOR, !BWD> xc[U][NV];  // forward: x is read with non-temporal loads
+        Chunk<T, VEC, VECTOR> dc[U][NV];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int r = min(rbase + u * NSLOT, r1 - 1);  // a row that exists; masked below if past the end
