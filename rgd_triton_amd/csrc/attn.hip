@@ -34,7 +34,8 @@ int fwd_blocks_per_cu(int dpad, bool bias) { return (dpad <= 64 && !bias) ? 3 : 
 size_t fwd_part_bytes(int dpad) { return (size_t)ATTN_BM * dpad * sizeof(float) + (size_t)ATTN_BM * 2 * sizeof(float); }
 
 // resident workgroups per compute unit of the backward kernels, and the bytes a part of a split item leaves
-int bwd_blocks_per_cu(int dpad) { return dpad <= 64 ? 2 : 1; }
+int bwd_blocks_per_cu(int dpad) { return dpad <= 64 ? 2 : 1; }           // dK/dV kernel
+int dq_blocks_per_cu(int dpad) { return (dpad <= 64 || dpad == 128) ? 2 : 1; }  // dQ kernel (32-key tiles at 128)
 size_t bwd_part_bytes(int dpad, int tensors) { return (size_t)tensors * BWD_BM * dpad * sizeof(float); }
 size_t bwd_delta_bytes(int64_t B, int64_t H, int64_t Tq) { return (size_t)(B * H * rgd_attn_seqlen_q_rounded(Tq)) * sizeof(float); }
 
@@ -212,8 +213,8 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
         const int64_t items = (int64_t)p.nblk * B * H;
         AttnSplit plan;
         if (may_split)
-            plan = attn_split_plan(items, rgd_num_cus(), per_cu, (int)((Tk + 63) / 64), bwd_part_bytes(dpad, 1), part_room,
-                                   kBwdSplit);
+            plan = attn_split_plan(items, rgd_num_cus(), dq_blocks_per_cu(dpad), (int)((Tk + 63) / 64),
+                                   bwd_part_bytes(dpad, 1), part_room, kBwdSplit);
         p.split_full = plan.full;
         p.split_s = plan.s;
         p.part = part_base;

@@ -91,21 +91,26 @@ __device__ __forceinline__ void store_row16(T* row, int col, int D, bool vec, co
 // ------------------------------------------------------------------------------------------------
 // dQ kernel
 // ------------------------------------------------------------------------------------------------
+#ifndef RGD_DQ_BN128
+#define RGD_DQ_BN128 32
+#endif
 template <int DPAD> struct DqSmem {
-    static constexpr int BN = 64;
+    // keys per tile: 32 at d = 128, where the smaller staging and logit registers let two wavefronts share a SIMD
+    static constexpr int BN = DPAD == 128 ? RGD_DQ_BN128 : 64;
     static constexpr int TILE = BN * BwdTile<DPAD>::S;
     static constexpr size_t BYTES = 2 * 2 * TILE * 2;  // K and V, double buffered
 };
 
 template <typename T, int DPAD, int BIAS>
-__global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dq_kernel(const AttnBwdParams p) {
+__global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32) ? 2 : 1) void attn_bwd_dq_kernel(const AttnBwdParams p) {
     constexpr bool HAS_BIAS = BIAS != BIAS_OFF;
     typedef typename BiasElem<T, BIAS>::type TB;
     typedef Mfma<T> MM;
     constexpr int BN = DqSmem<DPAD>::BN;
+    constexpr int NKB = BN / 32;  // 32-key halves per tile
     // starting the dP accumulators from -delta takes 16 registers; the bias variants at two wavefronts per
     // SIMD have none to spare and subtract delta per element instead
-    constexpr bool DP_INIT = BIAS == BIAS_OFF || DPAD > 64;
+    constexpr bool DP_INIT = BIAS == BIAS_OFF || (DPAD > 64 && DqSmem<DPAD>::BN == 64);
     constexpr int ST = BwdTile<DPAD>::S;
     constexpr int TILE = DqSmem<DPAD>::TILE;
     constexpr int NC = DPAD / 16;
@@ -216,7 +221,7 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dq_k
     const int a_off = mfma_row_perm(li) * ST + g * 8;
     const int tr_off = ((lane & 15) >> 2) * ST + mfma_row_perm(((lane >> 4) & 1) * 16 + (lane & 3) * 4) + g * 16 * ST;
     const TB* bias_row = nullptr;
-    BiasRuns<TB> bias_cur, bias_nxt;  // fetched one tile ahead of use
+    BiasRuns<TB, NKB> bias_cur, bias_nxt;  // fetched one tile ahead of use
     if constexpr (HAS_BIAS) {
         bias_row = static_cast<const TB*>(p.bias.ptr) + b * p.bias.sb + h * p.bias.sh + (int64_t)q_ld * p.bias.sn;
         if (t_begin < t_end) bias_cur.load(bias_row, t_begin * BN, g, p.Tk, p.bias_vec && (t_begin + 1) * BN <= p.Tk);
@@ -230,14 +235,14 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dq_k
             issue_loads(j + 1);
             if constexpr (HAS_BIAS) bias_nxt.load(bias_row, key0 + BN, g, p.Tk, p.bias_vec && key0 + 2 * BN <= p.Tk);
         }
-        float bias_v[2][16];
+        float bias_v[NKB][16];
         if constexpr (HAS_BIAS) bias_cur.decode(bias_v);
         const T* ks = ks_base + buf * TILE + a_off;
         const T* vs = vs_base + buf * TILE + a_off;
         // the dP accumulators start from -delta, so that product comes out as dP - delta
-        f32x16 s[2], dp[2];
+        f32x16 s[NKB], dp[NKB];
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
+        for (int kb = 0; kb < NKB; ++kb) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) s[kb][v] = 0.f;
             if constexpr (DP_INIT) {
@@ -256,7 +261,7 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dq_k
         }
         // t = logit - lse (log2 domain)
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+        for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 if constexpr (HAS_BIAS)
@@ -267,16 +272,16 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dq_k
         const bool diag = p.causal && (key0 + BN - 1 > qb * BWD_BM + wave * 32);
         if (tail || diag) {
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+            for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     const int key = key0 + kb * 32 + g * 16 + v;
                     if (key >= p.Tk || (p.causal && key > q_row)) s[kb][v] = -INFINITY;
                 }
         }
-        uint32_t dsk[2][8];
+        uint32_t dsk[NKB][8];
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+        for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
             for (int v = 0; v < 16; v += 2) {
                 const float p0 = __builtin_amdgcn_exp2f(s[kb][v]);
@@ -289,7 +294,7 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? 2 : 1) void attn_bwd_dq_k
         // dQ^T += K^T . dS^T
         const T* kt = ks_base + buf * TILE + tr_off;
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
+        for (int t = 0; t < 2 * NKB; ++t) {
             const int kb = t >> 1, jj = t & 1;
             const u32x4 raw = {dsk[kb][jj * 4 + 0], dsk[kb][jj * 4 + 1], dsk[kb][jj * 4 + 2], dsk[kb][jj * 4 + 3]};
             const typename MM::V8 bop = as_v8<T>(raw);

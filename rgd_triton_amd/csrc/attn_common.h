@@ -79,17 +79,17 @@ enum { BIAS_OFF = 0, BIAS_SAME = 1, BIAS_F32 = 2 };
 template <typename T, int BIAS> struct BiasElem { typedef T type; };
 template <typename T> struct BiasElem<T, BIAS_F32> { typedef float type; };
 
-// Raw bias of one lane for one 64-key tile in the "query per lane" layout: two runs of 16 contiguous
-// keys (key0 + 32*kb + 16*g ...).  load() only issues the memory reads, so it can run a whole tile
+// Raw bias of one lane for one tile of 32*NKB keys in the "query per lane" layout: NKB runs of 16
+// contiguous keys (key0 + 32*kb + 16*g ...).  load() only issues the memory reads, so it can run a whole tile
 // ahead of decode(); the registers hold the undecoded bits (8 VGPRs for a 16-bit bias).
-template <typename TB> struct BiasRuns {
+template <typename TB, int NKB = 2> struct BiasRuns {
     static constexpr int NV = 16 * sizeof(TB) / 16;  // 16-byte vectors per run
-    u32x4 raw[2][NV];
+    u32x4 raw[NKB][NV];
 
-    // row: &bias[b, h, q, 0].  fast = the run is 16-byte aligned and all 64 keys of the tile exist.
+    // row: &bias[b, h, q, 0].  fast = the run is 16-byte aligned and all keys of the tile exist.
     __device__ __forceinline__ void load(const TB* __restrict__ row, int key0, int g, int Tk, bool fast) {
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
+        for (int kb = 0; kb < NKB; ++kb) {
             const int first = key0 + kb * 32 + g * 16;
             if (fast) {
                 const u32x4* src = reinterpret_cast<const u32x4*>(row + first);
@@ -110,9 +110,9 @@ template <typename TB> struct BiasRuns {
 #pragma unroll
         for (int e = 0; e < 16; ++e) out[e] = static_cast<float>(tmp[e]);
     }
-    __device__ __forceinline__ void decode(float (&out)[2][16]) const {
+    __device__ __forceinline__ void decode(float (&out)[NKB][16]) const {
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
+        for (int kb = 0; kb < NKB; ++kb) {
             TB tmp[16];
             __builtin_memcpy(tmp, &raw[kb][0], sizeof(tmp));
 #pragma unroll
@@ -144,19 +144,6 @@ __device__ __forceinline__ typename Mfma<T>::V8 load_a_transposed(const T* tile,
     const u32x2 hi = lds_read_tr<T>(p + 4 * stride);
     const u32x4 raw = {lo[0], lo[1], hi[0], hi[1]};
     return as_v8<T>(raw);
-}
-
-// sum of the two 16-bit values of a packed pair, accumulated in fp32 (v_dot2c_f32_{bf16,f16} with ones)
-template <typename T> __device__ __forceinline__ float add_pair(uint32_t packed, float acc);
-template <> __device__ __forceinline__ float add_pair<bf16_t>(uint32_t packed, float acc) {
-    typedef bf16_t V2 __attribute__((ext_vector_type(2)));
-    const V2 ones = {(bf16_t)1.0f, (bf16_t)1.0f};
-    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(V2, packed), ones, acc, false);
-}
-template <> __device__ __forceinline__ float add_pair<f16_t>(uint32_t packed, float acc) {
-    typedef f16_t V2 __attribute__((ext_vector_type(2)));
-    const V2 ones = {(f16_t)1.0f, (f16_t)1.0f};
-    return __builtin_amdgcn_fdot2(__builtin_bit_cast(V2, packed), ones, acc, false);
 }
 
 // Workgroup ids are handed to the 8 XCDs round-robin and every XCD has its own L2.  This maps the
