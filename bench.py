@@ -12,7 +12,7 @@ independent buffer sets (4 x 268 MB) are used in rotation so that no step finds 
 
 Prints ONE JSON line: value = algorithmic GB/s of the whole step, `roofline` for the dominant
 kernel (the backward) from HIP events recorded around every launch inside the timed region,
-`cpu_baseline` = the CPU oracle timed on this host on a bounded sample, and `extra` with the other
+(minus the measured cost of an event), `cpu_baseline` = the CPU oracle timed on this host on a bounded sample, and `extra` with the other
 BASELINE configurations (attention TFLOP/s, RMSNorm2 / head LayerNorm GB/s) and the Module-API timing.
 """
 import argparse
@@ -59,7 +59,8 @@ def event_ms(pairs):
 
 def timed_loop(torch, step_fns, steps, warmup):
     """step_fns: list of callables (one per buffer set), each returns nothing and launches
-    [fwd, bwd] given an event recorder.  Returns (wall ms per step, fwd ms list, bwd ms list)."""
+    [fwd, bwd] given an event recorder.  Returns (wall ms per step, event span ms per step, fwd ms list,
+    bwd ms list, event-to-event gap ms)."""
     n = len(step_fns)
     for i in range(warmup):
         step_fns[i % n](None)
@@ -77,16 +78,19 @@ def timed_loop(torch, step_fns, steps, warmup):
     gpu_span = e0.elapsed_time(e1) / steps
     # the same steps again with an event after every launch: per-kernel durations for the roofline
     # (an event between two launches costs a few microseconds of stream time, which is why this is a
-    # separate pass and not the one `value` comes from)
+    # separate pass and not the one `value` comes from).  A fourth event recorded straight after the third
+    # measures that cost (event to event with nothing between); it is subtracted from both intervals.
     evs = []
     for i in range(steps):
-        rec = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+        rec = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
         step_fns[(i + steps) % n](rec)
+        rec[3].record()
         evs.append(rec)
     torch.cuda.synchronize()
-    fwd = [e[0].elapsed_time(e[1]) for e in evs]
-    bwd = [e[1].elapsed_time(e[2]) for e in evs]
-    return wall, gpu_span, fwd, bwd
+    gap = statistics.median(e[2].elapsed_time(e[3]) for e in evs)
+    fwd = [e[0].elapsed_time(e[1]) - gap for e in evs]
+    bwd = [e[1].elapsed_time(e[2]) - gap for e in evs]
+    return wall, gpu_span, fwd, bwd, gap
 
 
 def make_ln_rope_sets(torch, nsets, B=8, T=2048, H=16, D=64, R=32, seed=1002):
@@ -379,7 +383,7 @@ def main():
     B, T, H, D = 8, 2048, 16, 64
     pe, sets = make_ln_rope_sets(torch, 4, B, T, H, D)
     fns = ln_rope_steps(torch, pe, sets)
-    wall_ms, gpu_ms, fwd, bwd = timed_loop(torch, fns, args.steps, args.warmup)
+    wall_ms, gpu_ms, fwd, bwd, event_gap = timed_loop(torch, fns, args.steps, args.warmup)
     step_bytes = 5 * 2 * B * T * H * D * 2          # fwd: read x, write y; bwd: read x, dy, write dx (q and k)
     bwd_bytes = 3 * 2 * B * T * H * D * 2
     fwd_bytes = 2 * 2 * B * T * H * D * 2
@@ -401,6 +405,7 @@ def main():
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get("ln_rope_bwd_c2"),
                      "algorithmic_bytes_per_launch": bwd_bytes, "avg_launch_ms": round(bwd_avg, 5),
+                     "event_gap_ms_subtracted": round(event_gap, 5),
                      "fwd_kernel": {"achieved": round(fwd_bytes / fwd_avg / 1e6, 1), "avg_launch_ms": round(fwd_avg, 5),
                                     "frac": round(fwd_bytes / fwd_avg / 1e6 / HBM_PEAK_GBS, 4)}},
         "timing": {"wall_ms_per_step": round(wall_ms, 5), "gpu_event_span_ms_per_step": round(gpu_ms, 5)},
