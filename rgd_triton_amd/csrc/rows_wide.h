@@ -223,6 +223,132 @@ __global__ __launch_bounds__(NW * 64) void wide_rows_kernel(const WideParams p) 
     }
 }
 
+// Rows beyond the register-resident limit: a workgroup of 256 lanes owns one row at a time and streams over it
+// twice, lane t handling the chunks t, t+256, t+512, ... of VEC elements: the first pass accumulates the
+// row statistics, the second re-reads x (and dy, w) -- the row was just read, so this comes from L2 -- and
+// writes the result.  Only the dw sums of the RMSNorm backward stay in registers (NKW chunks per lane, a
+// compile-time bound; 0 when there is no dw); since every channel belongs to exactly one lane of the
+// workgroup, the block's partial dw row is written straight from them.
+template <typename T, int OP, bool BWD, int VEC, bool VECTOR, int NKW>
+__global__ __launch_bounds__(256) void wide_stream_kernel(const WideParams p) {
+    __shared__ float s_red[2][2][4];  // [parity][statistic][wavefront]
+    constexpr bool HAS_W = (OP == WIDE_RMS);
+    const int which = (int)blockIdx.x >= p.h[0].nchunks ? 1 : 0;
+    const WideHalf& h = p.h[which];
+    const int chunk = blockIdx.x - (which ? p.h[0].nchunks : 0);
+    const int b = blockIdx.y;
+    const int C = h.C;
+    const int r0 = chunk * p.rows_per_chunk;
+    const int r1 = min(h.T, r0 + p.rows_per_chunk);
+    const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6;
+    const int nk = (C + 256 * VEC - 1) / (256 * VEC);  // chunks per lane
+
+    const T* xb = static_cast<const T*>(h.x) + (int64_t)b * h.sx_b;
+    const T* db = BWD ? static_cast<const T*>(h.dy) + (int64_t)b * h.sd_b : nullptr;
+    T* yb = static_cast<T*>(h.y) + (int64_t)b * h.sy_b;
+    const char* wp = HAS_W ? static_cast<const char*>(h.w) + (int64_t)b * h.sw_b * (h.w_dtype == RGD_F32 ? 4 : 2) : nullptr;
+    const bool w_vec = VECTOR && h.w_vec;
+    auto load_w = [&](int first, float (&w)[VEC]) {
+        if (w_vec)
+            load_chunk_dyn<VEC, VECTOR>(wp, h.w_dtype, first, C, w);
+        else
+            load_chunk_dyn<VEC, false>(wp, h.w_dtype, first, C, w);
+    };
+
+    constexpr int NACC = NKW > 0 ? NKW : 1;
+    float dwacc[NACC][VEC];
+#pragma unroll
+    for (int k = 0; k < NACC; ++k)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) dwacc[k][e] = 0.f;
+
+    for (int r = r0; r < r1; ++r) {
+        const T* xr = xb + (int64_t)r * h.sx_n;
+        const T* dr = BWD ? db + (int64_t)r * h.sd_n : nullptr;
+        // ---- pass 1: sum x^2 (and sum x*dy*w) ----
+        float ss = 0.f, sd = 0.f;
+        for (int k = 0; k < nk; ++k) {
+            const int first = (k * 256 + tid) * VEC;
+            float xv[VEC], dv[VEC], wv[VEC];
+            load_chunk<T, VEC, VECTOR>(xr, first, C, xv);
+            if constexpr (BWD) {
+                load_chunk<T, VEC, VECTOR>(dr, first, C, dv);
+                if constexpr (HAS_W) load_w(first, wv);
+            }
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                ss += xv[e] * xv[e];
+                if constexpr (BWD) sd += xv[e] * (HAS_W ? dv[e] * wv[e] : dv[e]);
+            }
+        }
+        ss = group_reduce<64>(ss);
+        if constexpr (BWD) sd = group_reduce<64>(sd);
+        const int par = (r - r0) & 1;
+        if (lane == 0) {
+            s_red[par][0][wave] = ss;
+            if constexpr (BWD) s_red[par][1][wave] = sd;
+        }
+        __syncthreads();
+        ss = (s_red[par][0][0] + s_red[par][0][1]) + (s_red[par][0][2] + s_red[par][0][3]);
+        if constexpr (BWD) sd = (s_red[par][1][0] + s_red[par][1][1]) + (s_red[par][1][2] + s_red[par][1][3]);
+        float rn;  // rrms or rlen
+        if constexpr (OP == WIDE_RMS) {
+            rn = rsqrtf(ss * h.inv_c + p.eps);
+        } else {
+            const float len = sqrtf(ss);
+            rn = len < p.eps ? 1.0f / p.eps : 1.0f / len;
+        }
+        const float inner = OP == WIDE_RMS ? sd * rn * h.inv_c : sd * rn;
+        // ---- pass 2: results ----
+        T* yr = yb + (int64_t)r * h.sy_n;
+        auto body = [&](int k, float (&acc)[VEC]) {
+            const int first = (k * 256 + tid) * VEC;
+            float xv[VEC], dv[VEC], wv[VEC], out[VEC];
+            load_chunk<T, VEC, VECTOR>(xr, first, C, xv);
+            if constexpr (BWD) load_chunk<T, VEC, VECTOR>(dr, first, C, dv);
+            if constexpr (HAS_W) load_w(first, wv);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                if constexpr (!BWD) {
+                    out[e] = HAS_W ? xv[e] * rn * wv[e] : xv[e] * rn;
+                } else {
+                    const float xh = xv[e] * rn;
+                    const float gr = HAS_W ? dv[e] * wv[e] : dv[e];
+                    out[e] = (gr - xh * inner) * rn;
+                    if constexpr (NKW > 0) acc[e] += xh * dv[e];
+                }
+            }
+            store_chunk<T, VEC, VECTOR>(yr, first, C, out);
+        };
+        if constexpr (NKW > 0) {
+#pragma unroll
+            for (int k = 0; k < NKW; ++k)
+                if (k < nk) body(k, dwacc[k]);
+        } else {
+            for (int k = 0; k < nk; ++k) body(k, dwacc[0]);
+        }
+    }
+
+    if constexpr (NKW > 0) {
+        const int wgt = h.w_shared ? 0 : b;
+        const int idx = h.w_shared ? b * h.nchunks + chunk : chunk;
+        void* dw_row = static_cast<char*>(h.dw) + (int64_t)wgt * h.sdw_b * (h.w_dtype == RGD_F32 ? 4 : 2);
+        float* mine = h.part + ((int64_t)wgt * h.nleaf + idx) * C;
+#pragma unroll
+        for (int k = 0; k < NKW; ++k)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const int c = (k * 256 + tid) * VEC + e;
+                if (c < C) {
+                    if (h.nleaf == 1)
+                        store_dyn(dw_row, h.w_dtype, c, dwacc[k][e]);
+                    else
+                        mine[c] = dwacc[k][e];
+                }
+            }
+    }
+}
+
 // host-side description of one (B,T,C) half handed to the launchers
 struct WideHalfArgs {
     int64_t T = 0, C = 0;
@@ -246,7 +372,10 @@ struct WideConfig {
     bool bwd;
     int G, NV, WPR;
     bool vector;
+    bool stream;  // rows beyond the register-resident limit: wide_stream_kernel
 };
+// chunks of dw sums a lane of the streaming RMSNorm backward holds: at most 64 fp32 accumulators
+constexpr int wide_stream_nkw(int vec) { return vec >= 4 ? 64 / vec : 16; }
 // compile-time launch shape shared by the kernel instantiations and the host-side grid computation
 // rows a lane group has in flight at once, by the elements of one row a lane holds (nv chunks of vec)
 constexpr int wide_unroll(bool bwd, int nv, int vec) {

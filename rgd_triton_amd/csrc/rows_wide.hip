@@ -135,13 +135,20 @@ int wide_launch(const char* name, int op, bool bwd, int64_t B, const WideHalfArg
                     break;
                 }
         }
-        RGD_REQUIRE(cfg.NV != 0, RGD_ERR_UNSUPPORTED,
-                    "%s: rows of %lld elements exceed the register-resident limit (%d)", name, (long long)maxC,
-                    256 * max_epl);
     }
-    const int NW = wide_waves(op, bwd);
-    const int U = wide_unroll(bwd, cfg.NV, vec);
-    const int row_quantum = NW * (64 / cfg.G) / cfg.WPR * U;
+    cfg.stream = cfg.NV == 0;  // too wide for registers: the two-pass streaming kernel
+    if (cfg.stream) {
+        const int64_t dw_limit = (int64_t)256 * wide_stream_nkw(vec) * vec;  // dw sums stay in registers
+        RGD_REQUIRE(!(has_w && bwd) || maxC <= dw_limit, RGD_ERR_UNSUPPORTED,
+                    "%s: rows of %lld elements exceed the limit of the backward (%lld)", name, (long long)maxC,
+                    (long long)dw_limit);
+        cfg.G = 64;
+        cfg.NV = 1;
+        cfg.WPR = 4;
+    }
+    const int NW = cfg.stream ? 4 : wide_waves(op, bwd);
+    const int U = cfg.stream ? 1 : wide_unroll(bwd, cfg.NV, vec);
+    const int row_quantum = cfg.stream ? 1 : NW * (64 / cfg.G) / cfg.WPR * U;
     const bool tree = has_w && bwd;
     const int64_t target = (int64_t)rgd_num_cus() * (tree ? DW_BLOCKS_PER_CU : BLOCKS_PER_CU);
     int64_t rpc = (total_rows + target - 1) / target;
@@ -207,7 +214,8 @@ int wide_launch(const char* name, int op, bool bwd, int64_t B, const WideHalfArg
     RGD_REQUIRE(grid_x < (1ll << 31), RGD_ERR_UNSUPPORTED, "%s: grid too large", name);
 
     const dim3 grid((unsigned)grid_x, (unsigned)B, 1);
-    const size_t lds = tree ? (size_t)(NW / cfg.WPR) * maxC * sizeof(float) : 0;  // one row of sums per wavefront group
+    // one row of dw sums per wavefront group (the streaming kernel writes its sums from registers)
+    const size_t lds = (tree && !cfg.stream) ? (size_t)(NW / cfg.WPR) * maxC * sizeof(float) : 0;
     RGD_REQUIRE(lds <= 64 * 1024, RGD_ERR_UNSUPPORTED, "%s: row too wide for the dw staging buffer", name);
     hipStream_t s = static_cast<hipStream_t>(stream);
     int rc;

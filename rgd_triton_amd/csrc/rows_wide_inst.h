@@ -52,8 +52,25 @@ static int wide_dispatch_shape(const WideConfig& c, const WideParams& p, dim3 gr
     return RGD_ERR_UNSUPPORTED;
 }
 
+template <typename T, int OP, bool BWD, bool VECTOR>
+static int wide_launch_stream(const WideParams& p, dim3 grid, hipStream_t s) {
+    constexpr int VEC = VECTOR ? 16 / (int)sizeof(T) : 2;
+    constexpr int NKW = (OP == WIDE_RMS && BWD) ? wide_stream_nkw(VEC) : 0;
+    hipLaunchKernelGGL((wide_stream_kernel<T, OP, BWD, VEC, VECTOR, NKW>), grid, dim3(256), 0, s, p);
+    return 0;
+}
+
 template <typename T>
 int wide_dispatch(const WideConfig& c, const WideParams& p, dim3 grid, size_t lds, hipStream_t s) {
+#define WIDE_STREAM(OP_, BWD_)                                                            \
+    if (c.stream && c.op == OP_ && c.bwd == BWD_)                                         \
+        return c.vector ? wide_launch_stream<T, OP_, BWD_, true>(p, grid, s)              \
+                        : wide_launch_stream<T, OP_, BWD_, false>(p, grid, s);
+    WIDE_STREAM(WIDE_RMS, false)
+    WIDE_STREAM(WIDE_RMS, true)
+    WIDE_STREAM(WIDE_L2, false)
+    WIDE_STREAM(WIDE_L2, true)
+#undef WIDE_STREAM
 #define WIDE_OP(OP_, BWD_)                                                                      \
     if (c.op == OP_ && c.bwd == BWD_)                                                           \
         return c.vector ? wide_dispatch_shape<T, OP_, BWD_, true>(c, p, grid, lds, s)           \

@@ -25,6 +25,22 @@ def test_l2_norm(T, C, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("C", [16392, 20001, 40000])
+def test_l2_norm_streamed_rows(C, dtype):
+    """rows beyond the register-resident limit: two-pass streaming kernel, any width"""
+    from rgd_triton_amd import triton_norm_func_fn
+
+    g = gen(C)
+    x = randn(g, 2, 23, C, dtype=dtype, scale=100.0)
+    dy = randn(g, 2, 23, C, dtype=dtype)
+    xg = to_gpu(x, requires_grad=True)
+    y = triton_norm_func_fn(xg, 1e-6)
+    (dx,) = torch.autograd.grad(y, xg, dy.to("cuda"))
+    assert_close(y, oracle.l2_fwd(x, 1e-6), dtype, name="y")
+    assert_close_allow_inf(dx, oracle.l2_bwd(dy, x, 1e-6), dtype, name="dx")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_l2_clamped_rows(dtype):
     """rows shorter than eps (including all-zero rows) take the 1/eps branch, forward and backward"""
     from rgd_triton_amd import L2Normalize

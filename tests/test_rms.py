@@ -54,13 +54,29 @@ def test_rms_norm_wide_rows(T, unique_bw, C, dtype):
     assert_close(dw, dw_ref, dtype, "rms", "dw", atol_scale=3 * rows * C ** 0.5)
 
 
-def test_rms_too_wide_is_rejected():
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("C,unique_bw", [(8200, False), (10001, False), (12288, True), (16384, False)])
+def test_rms_norm_streamed_rows(C, unique_bw, dtype):
+    """Rows beyond the register-resident limit take the two-pass streaming kernel (the reference loops over
+    channel blocks for any C); its backward holds the dw sums of 16384 channels (8192 unaligned) at most."""
     from rgd_triton_amd import triton_rms_func_fn
 
-    x = torch.zeros(1, 4, 8192 + 8, device="cuda", dtype=torch.bfloat16)
-    w = torch.ones(8192 + 8, device="cuda", dtype=torch.bfloat16)
-    with pytest.raises(RuntimeError, match="register-resident"):
-        triton_rms_func_fn(x, w, 1e-6)
+    B, T = 2, 37
+    if C % 8 and C > 8192:  # odd width: forward only, the backward must refuse
+        g = gen(C)
+        x = randn(g, B, T, C, dtype=dtype)
+        w = (1 + 0.1 * torch.randn(C, generator=g)).to(dtype)
+        xg, wg = to_gpu(x, w, requires_grad=True)
+        y = triton_rms_func_fn(xg, wg, 1e-6)
+        assert_close(y, oracle.rms_fwd(x, w, 1e-6), dtype, "rms", "y")
+        with pytest.raises(RuntimeError, match="exceed the limit of the backward"):
+            torch.autograd.grad(y, (xg, wg), torch.ones_like(y))
+        return
+    (y, dx, dw), (y_ref, dx_ref, dw_ref) = _run(B, T, C, dtype, unique_bw, seed=C)
+    assert_close(y, y_ref, dtype, "rms", "y")
+    assert_close(dx, dx_ref, dtype, "rms", "dx")
+    rows = T if unique_bw else B * T
+    assert_close(dw, dw_ref, dtype, "rms", "dw", atol_scale=3 * rows * C ** 0.5)
 
 
 @pytest.mark.parametrize("T", [1, 3, 31, 97, 200, 1025])
@@ -111,7 +127,7 @@ def test_rms_strided_views():
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("C,T", [(384, 239), (1023, 113), (1536, 512), (6144, 67)])
+@pytest.mark.parametrize("C,T", [(384, 239), (1023, 113), (1536, 512), (6144, 67), (12288, 19)])
 def test_rms_deterministic(C, T, dtype):
     """The reference's race test (tests/test_rms.py:193-246): batch 60, repeated runs must give
     bit-identical y, dx and dw."""
