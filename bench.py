@@ -42,8 +42,9 @@ MEASURED_TRAFFIC = {
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=1000,
+                    help="untimed steps; the GPU needs tens of milliseconds of work to reach its steady clocks")
     ap.add_argument("--skip-extra", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--only", default="", help="run only this extra workload (for profiling)")
@@ -157,7 +158,21 @@ def cpu_baseline_ln_rope(torch, B=2, T=2048, H=16, D=64, R=32, reps=3):
 # ------------------------------------------------------------------------------------------------
 # extra workloads (reported under "extra", not the headline value)
 # ------------------------------------------------------------------------------------------------
+def spin_up(torch, fn, seconds=0.06):
+    """Untimed launches for `seconds`: after an idle spell (allocation, input generation on the host) the GPU
+    needs tens of milliseconds of work before its clocks reach their steady state, and a kernel timed during
+    that ramp reads 5-20 % slow."""
+    t0 = time.perf_counter()
+    i = 0
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(8):
+            fn(i)
+            i += 1
+        torch.cuda.synchronize()
+
+
 def time_api(torch, fn, iters=30, warmup=5):
+    spin_up(torch, lambda i: fn())
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -213,7 +228,24 @@ def attention_case(torch, name, B, T, H, D, dtype, bias_kind, iters=20):
                                 t["dq"], t["dk"], t["dv"], code, 0, scale, ws.data_ptr(), ws.numel(), st) == 0, \
             lib.rgd_last_error()
 
-    f_ms, b_ms = time_api(torch, fwd, iters, 3), time_api(torch, bwd, iters, 3)
+    # forward and backward alternate as in a training step; the clocks are brought to their steady state first
+    def step(_):
+        fwd()
+        bwd()
+
+    spin_up(torch, step, 0.1)
+    evs = []
+    for _ in range(iters):
+        e = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+        e[0].record()
+        fwd()
+        e[1].record()
+        bwd()
+        e[2].record()
+        evs.append(e)
+    torch.cuda.synchronize()
+    f_ms = statistics.mean(e[0].elapsed_time(e[1]) for e in evs)
+    b_ms = statistics.mean(e[1].elapsed_time(e[2]) for e in evs)
     flops = 14.0 * B * H * T * T * D
     tot = f_ms + b_ms
     return {"workload": name, "fwd_ms": round(f_ms, 4), "bwd_ms": round(b_ms, 4),
@@ -225,6 +257,7 @@ def time_pair(torch, fwd, bwd, nsets, iters=60, warmup=8):
     """average ms of fwd(i) and of bwd(i) (i = buffer set), each timed as a run of back-to-back launches"""
     out = []
     for fn in (fwd, bwd):
+        spin_up(torch, lambda i: fn(i % nsets))
         for i in range(warmup):
             fn(i % nsets)
         torch.cuda.synchronize()
