@@ -19,7 +19,10 @@ enum { WIDE_RMS = 0, WIDE_L2 = 1 };
 #ifndef RGD_WIDE_EPL_U2
 #define RGD_WIDE_EPL_U2 16  // backward: two rows in flight up to this many elements per lane
 #endif
-constexpr int WIDE_RED_WAVES = 8;  // wavefronts of a reduce block; each adds every 8th partial row
+#ifndef RGD_WIDE_RED_WAVES
+#define RGD_WIDE_RED_WAVES 16
+#endif
+constexpr int WIDE_RED_WAVES = RGD_WIDE_RED_WAVES;  // wavefronts of a reduce block; wavefront w adds partial rows w, w+WAVES, ...
 
 struct WideHalf {
     const void* x;

@@ -28,7 +28,7 @@ size_t half_bound(int64_t B, int64_t T, int64_t target) {
 }
 
 // dw[weight][c] = sum over the partial rows of that weight, in a fixed order: wavefront w of the block adds
-// rows w, w+8, w+16, ... for 64 consecutive channels, then the 8 wavefront sums are added in index order.
+// rows w, w+WAVES, w+2*WAVES, ... for 64 consecutive channels, then the wavefront sums are added in index order.
 __global__ __launch_bounds__(WIDE_RED_WAVES * 64) void wide_dw_reduce_kernel(const WideParams p) {
     __shared__ float s_sum[WIDE_RED_WAVES][64];
     const int which = (int)blockIdx.x >= p.h[0].red_blocks ? 1 : 0;
@@ -42,13 +42,15 @@ __global__ __launch_bounds__(WIDE_RED_WAVES * 64) void wide_dw_reduce_kernel(con
     float acc = 0.f;
     if (c < h.C) {
         int r = wave;
+        // the partial rows were written by other compute units moments ago, so every read is a trip to the
+        // memory side: eight independent reads in flight per lane, added in row order
 #pragma unroll 1
-        for (; r + 3 * WIDE_RED_WAVES < h.nleaf; r += 4 * WIDE_RED_WAVES) {  // four loads in flight
-            const float v0 = src[(int64_t)r * h.C];
-            const float v1 = src[(int64_t)(r + WIDE_RED_WAVES) * h.C];
-            const float v2 = src[(int64_t)(r + 2 * WIDE_RED_WAVES) * h.C];
-            const float v3 = src[(int64_t)(r + 3 * WIDE_RED_WAVES) * h.C];
-            acc = (((acc + v0) + v1) + v2) + v3;
+        for (; r + 7 * WIDE_RED_WAVES < h.nleaf; r += 8 * WIDE_RED_WAVES) {
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = src[(int64_t)(r + i * WIDE_RED_WAVES) * h.C];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc += v[i];
         }
         for (; r < h.nleaf; r += WIDE_RED_WAVES) acc += src[(int64_t)r * h.C];
     }
