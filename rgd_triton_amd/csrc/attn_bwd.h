@@ -351,20 +351,37 @@ template <int DPAD, int NSUB> struct DkvSmem {
 // 16 bias values of one key column (16 consecutive rows of the bias matrix) in the "key per lane" layout.
 // load() only issues the reads so it can run a tile ahead of decode().  `tile_rows` points at the first
 // bias row of the query tile and is the same for the whole wavefront, `lane_off` is this lane's element
-// offset from there (its key column plus 16*g rows), so every read is a wavefront-uniform base plus a
-// 32-bit lane offset and needs no per-lane address arithmetic.  A ragged last tile (rows_ok false) reads
+// offset from there (its key column plus 16*g rows).  The reads are buffer loads: one descriptor on the tile,
+// the lane offset in ONE register for all rows, and the row offset v*sn in a scalar register, so no per-lane
+// address arithmetic or address registers per row are needed.  A ragged last tile (rows_ok false) reads
 // the last existing row instead of rows >= Tq; the caller masks those.
 template <typename TB> struct BiasColumn {
     TB raw[16];
     __device__ __forceinline__ void load(const TB* __restrict__ tile_rows, int64_t sn, uint32_t lane_off, int row0,
                                          int Tq, bool rows_ok) {
         if (rows_ok) {
+            // raw buffer over the tile: offsets stay below 2^31 bytes because row strides are below 2^24 elements
+            const __amdgpu_buffer_rsrc_t rsrc =
+                __builtin_amdgcn_make_buffer_rsrc(const_cast<TB*>(tile_rows), 0, 0xffffffffu, 0x00020000);
+            const uint32_t voff = lane_off * (uint32_t)sizeof(TB);
+            const uint32_t row_bytes = (uint32_t)sn * (uint32_t)sizeof(TB);
 #pragma unroll
-            for (int v = 0; v < 16; ++v) raw[v] = (tile_rows + v * sn)[lane_off];
+            for (int v = 0; v < 16; ++v) {
+                if constexpr (sizeof(TB) == 2) {
+                    const uint16_t bits = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rsrc, voff, v * row_bytes, 0);
+                    raw[v] = __builtin_bit_cast(TB, bits);
+                } else {
+                    const uint32_t bits = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc, voff, v * row_bytes, 0);
+                    raw[v] = __builtin_bit_cast(TB, bits);
+                }
+            }
         } else {
-            const TB* col = tile_rows + lane_off;  // rows_ok is false at most once per workgroup
+            // rows_ok is false at most once per workgroup.  `last` is the one per-lane quantity (written so that
+            // the loop around this call carries one value for this branch, not one per row).
+            const TB* col = tile_rows + lane_off;
+            const int last = Tq - 1 - row0;  // last existing row relative to this lane's first row (may be < 0)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) raw[v] = col[(int64_t)(min(row0 + v, Tq - 1) - row0) * sn];
+            for (int v = 0; v < 16; ++v) raw[v] = col[(int64_t)min(v, last) * sn];
         }
     }
     __device__ __forceinline__ void decode(float (&out)[16]) const {
