@@ -86,9 +86,8 @@ def _rms_scratch(x1, x2):
     T2, C2 = (x2.shape[1], x2.shape[2]) if x2 is not None else (0, 0)
     _hip.check(lib.rgd_rms_bwd_workspace(B, x1.shape[1], x1.shape[2], T2, C2, ctypes.byref(ws), ctypes.byref(ct)),
                "rgd_rms_bwd_workspace")
-    wbuf = _hip.scratch(x1.device, "rms_ws", ws.value)
-    cbuf = _hip.scratch(x1.device, "rms_ctr", ct.value, zero=True)
-    return wbuf, ws.value, cbuf, ct.value
+    # counter_bytes is 0 in this version of the library: the backward takes a null counter buffer
+    return _hip.scratch(x1.device, "rms_ws", ws.value), ws.value
 
 
 class RMS_Func(torch.autograd.Function):
@@ -123,11 +122,11 @@ class RMS_Func(torch.autograd.Function):
         if T == 0:
             dw.zero_()
             return dx, dw, None, None
-        wbuf, wsz, cbuf, csz = _rms_scratch(x, None)
+        wbuf, wsz = _rms_scratch(x, None)
         lib = _hip.lib()
         _hip.check(lib.rgd_rms_bwd(B, T, C, t3(dy), t3(x), t3(w, w_sb), t3(dx), t3(dw, 0 if shared else dw.stride(0)),
                                    int(shared), _hip.dtype_code(x.dtype), _hip.dtype_code(w.dtype), ctx.norm_eps,
-                                   wbuf.data_ptr(), wsz, cbuf.data_ptr(), csz, _hip.stream_ptr(x.device)), "rgd_rms_bwd")
+                                   wbuf.data_ptr(), wsz, None, 0, _hip.stream_ptr(x.device)), "rgd_rms_bwd")
         return dx, dw, None, None
 
 
@@ -175,14 +174,14 @@ class Fused_RMS_Func(torch.autograd.Function):
             dw1.zero_()
         if T2 == 0:
             dw2.zero_()
-        wbuf, wsz, cbuf, csz = _rms_scratch(x1, x2)
+        wbuf, wsz = _rms_scratch(x1, x2)
         lib = _hip.lib()
         _hip.check(lib.rgd_fused_rms_bwd(
             B, T1, C1, T2, C2,
             t3(dy1), t3(x1), t3(w1, sb1), t3(dx1), t3(dw1, 0 if s1 else dw1.stride(0)), int(s1),
             t3(dy2), t3(x2), t3(w2, sb2), t3(dx2), t3(dw2, 0 if s2 else dw2.stride(0)), int(s2),
             _hip.dtype_code(x1.dtype), _hip.dtype_code(w1.dtype), _hip.dtype_code(w2.dtype), ctx.norm_eps,
-            wbuf.data_ptr(), wsz, cbuf.data_ptr(), csz, _hip.stream_ptr(x1.device)), "rgd_fused_rms_bwd")
+            wbuf.data_ptr(), wsz, None, 0, _hip.stream_ptr(x1.device)), "rgd_fused_rms_bwd")
         return dx1, dx2, dw1, dw2, None, None
 
 

@@ -45,7 +45,9 @@ def test_error_paths_return_codes_without_a_gpu():
     assert b"Only support fp16, bf16, and fp32" in lib.rgd_last_error()
     assert lib.rgd_rms_fwd(1, 1, 8, None, t3, t3, 0, 0, 1e-6, None) == -1
     assert lib.rgd_l2_fwd(70000, 1, 8, t3, t3, 0, 1e-6, None) == -1           # batch beyond the grid limit
-    assert lib.rgd_rms_fwd(1, 4, 200000, t3, t3, t3, 0, 0, 1e-6, None) == -2     # row too wide for registers
+    # rows of any width stream through the forward; the backward (dw sums in registers) has a limit
+    assert lib.rgd_rms_bwd(1, 4, 200000, t3, t3, t3, t3, t3, 1, 0, 0, 1e-6, 0x1000, 1 << 30, None, 0, None) == -2
+    assert b"exceed the limit of the backward" in lib.rgd_last_error()
     assert lib.rgd_ln_qk_fwd(1, 1, 4, 4, 300, t4, t4, t4, t4, 0, 1e-6, None) == -1
     assert b"head dimensions up to 256" in lib.rgd_last_error()
     assert lib.rgd_rope_qk(1, 1, 4, 4, 160, t4, t4, t4, t4, 0x1000, 8, 32, 256, 32, 0, 4, 4, 0, 0, None) == -1
