@@ -91,7 +91,7 @@ __device__ __forceinline__ void load_chunk(const T* __restrict__ p, int first, i
     }
 }
 
-template <typename T, int N, bool VECTOR>
+template <typename T, int N, bool VECTOR, bool NT = false>
 __device__ __forceinline__ void store_chunk(T* __restrict__ p, int first, int limit, const float (&in)[N]) {
     if constexpr (VECTOR && (N * sizeof(T)) % 16 == 0) {
         constexpr int BYTES = N * sizeof(T);
@@ -106,7 +106,10 @@ __device__ __forceinline__ void store_chunk(T* __restrict__ p, int first, int li
                 for (int e = 0; e < EPV; ++e) tmp[e] = from_f32<T>(in[v * EPV + e]);
                 u32x4 raw;
                 __builtin_memcpy(&raw, tmp, 16);
-                vp[v] = raw;
+                if constexpr (NT)
+                    __builtin_nontemporal_store(raw, vp + v);
+                else
+                    vp[v] = raw;
             }
         }
     } else {
@@ -120,9 +123,9 @@ __device__ __forceinline__ void store_chunk(T* __restrict__ p, int first, int li
 // range reads the start of the row instead, which is always valid memory) and out-of-range elements are
 // zeroed by a select when the raw bits are decoded.  Issue every load() of an iteration first, then
 // decode(): the loads overlap and the wavefront waits once.
-// NT: non-temporal loads (data that is read once and not shared between workgroups).  Measured: they
-// shorten forward kernels (one input stream) by 7-12 % and lengthen backward kernels (two input streams) by
-// 15 %.
+// NT: non-temporal loads (data that is read once and not shared between workgroups).  Measured: on x they
+// shorten forward kernels by 7-12 % but take the rows out of the Infinity Cache, which a backward that
+// re-reads them soon pays for; on the upstream gradient of the backward kernels they gain 3-5 %.
 template <typename T, int N, bool VECTOR, bool NT = false> struct Chunk {
     static constexpr bool VEC = VECTOR && (N * sizeof(T)) % 16 == 0;
     static constexpr int NVEC = VEC ? (N * sizeof(T)) / 16 : 1;

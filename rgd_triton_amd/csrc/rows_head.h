@@ -58,9 +58,12 @@ __global__ __launch_bounds__(256) void head_rows_kernel(const HeadParams p) {
     const uint32_t row0 = (blockIdx.x - (which ? p.blocks_q : 0u)) * (uint32_t)(ROWS_PER_PASS * U) + wave * GPW + lane / G;
     const int D = p.D;
 
-    // plain (temporal) loads on purpose: non-temporal loads of x shorten the forward by 7 % but leave nothing
-    // of q, k in the Infinity Cache for a backward that follows soon, which then takes 17 % longer
-    Chunk<T, VEC, VECTOR> xc[U][NV], dc[U][NV];
+    // x: plain (temporal) loads on purpose.  Non-temporal loads of x shorten the forward by 7 % but leave nothing
+    // of q, k in the Infinity Cache for a backward that follows soon, which then takes 17 % longer; in the
+    // backward they slow the next forward by a third.  dy is read once and nothing else wants it: non-temporal
+    // (the forward+backward step gains 3 %).  Non-temporal stores change nothing.
+    Chunk<T, VEC, VECTOR> xc[U][NV];
+    Chunk<T, VEC, VECTOR, true> dc[U][NV];
     Chunk<TP, VEC, VECTOR> sc[U][NV], cc[U][NV];
     bool rotate[U];
     int lim[U];

@@ -97,7 +97,7 @@ __global__ __launch_bounds__(NW * 64) void wide_rows_kernel(const WideParams p) 
     for (int it = 0; it < iters; ++it) {
         const int rbase = r0 + slot + it * NSLOT * U;
         Chunk<T, VEC, VECTOR, !BWD> xc[U][NV];  // forward: x is read with non-temporal loads
-        Chunk<T, VEC, VECTOR> dc[U][NV];
+        Chunk<T, VEC, VECTOR, true> dc[U][NV];   // the upstream gradient is read once: non-temporal
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int r = min(rbase + u * NSLOT, r1 - 1);  // a row that exists; masked below if past the end
