@@ -33,9 +33,9 @@ MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # this file (profiles/), scaled by a copy kernel of known size; None until measured for a workload.
 MEASURED_TRAFFIC = {
-    # FETCH_SIZE 65767.0 KiB x 2.0 (copy calibration) + WRITE_SIZE 65536.0 KiB x 1.0, per launch of the
+    # FETCH_SIZE 65737.6 KiB x 2.0 (copy calibration) + WRITE_SIZE 65536.0 KiB x 1.0, per launch of the
     # LN+RoPE backward on this workload (profiles/head_rows_lnrope_config2.md)
-    "ln_rope_bwd_c2": 201799680,
+    "ln_rope_bwd_c2": 201739469,
 }
 
 
