@@ -135,8 +135,8 @@ def ln_rope_steps(torch, pe, sets, eps=1e-5):
     return fns
 
 
-def cpu_baseline_ln_rope(torch, B=2, T=2048, H=16, D=64, R=32, reps=3):
-    """The CPU oracle (oracle/rgd_oracle.py, PyTorch eager fp32) on a batch-2 slice of the workload."""
+def cpu_baseline_ln_rope(torch, B=8, T=2048, H=16, D=64, R=32, reps=3):
+    """The CPU oracle (oracle/rgd_oracle.py, PyTorch eager fp32) on the full workload, all host threads."""
     import rgd_oracle as oracle
 
     g = torch.Generator().manual_seed(1002)
@@ -158,6 +158,64 @@ def cpu_baseline_ln_rope(torch, B=2, T=2048, H=16, D=64, R=32, reps=3):
 # ------------------------------------------------------------------------------------------------
 # extra workloads (reported under "extra", not the headline value)
 # ------------------------------------------------------------------------------------------------
+
+def _cpu_time(fn, reps=2):
+    times = []
+    for i in range(reps + 1):
+        t0 = time.perf_counter()
+        fn()
+        if i:
+            times.append(time.perf_counter() - t0)
+    return statistics.median(times)
+
+
+def cpu_extra(torch, kind, **kw):
+    """The CPU oracle on a bounded sample of an extra workload (a few seconds each), timed beside the GPU figure."""
+    import rgd_oracle as oracle
+
+    g = torch.Generator().manual_seed(7)
+    cores = torch.get_num_threads()
+    if kind == "rms":
+        B, shapes, dtype = kw["B"], kw["shapes"], kw["dtype"]
+        xs = [torch.randn(B, T, C, generator=g).to(dtype) for T, C in shapes]
+        ds = [torch.randn(B, T, C, generator=g).to(dtype) for T, C in shapes]
+        ws = [(1 + 0.1 * torch.randn(C, generator=g)).to(dtype) for _, C in shapes]
+
+        def run():
+            for x, d, w in zip(xs, ds, ws):
+                oracle.rms_fwd(x, w)
+                oracle.rms_bwd(d, x, w)
+        t = _cpu_time(run)
+        nbytes = 5 * sum(x.numel() * x.element_size() for x in xs)
+        return {"value": round(nbytes / t / 1e9, 3), "unit": "GB/s", "ms": round(t * 1e3, 2), "cores": cores, "kind": "port",
+                "sample": "oracle rms_fwd+rms_bwd on the full workload"}
+    if kind == "head_ln":
+        B, T, H, D, dtype = kw["B"], kw["T"], kw["H"], kw["D"], kw["dtype"]
+        q, k, gq, gk = (torch.randn(1, T, H, D, generator=g).to(dtype) for _ in range(4))
+
+        def run():
+            for x, d in ((q, gq), (k, gk)):
+                oracle.head_ln_fwd(x)
+                oracle.head_ln_bwd(d, x)
+        t = _cpu_time(run)
+        nbytes = 5 * 2 * q.numel() * q.element_size()
+        return {"value": round(nbytes / t / 1e9, 3), "unit": "GB/s", "ms": round(t * 1e3, 2), "cores": cores, "kind": "port",
+                "sample": f"oracle head_ln_fwd+head_ln_bwd on one of {B} batch elements"}
+    if kind == "attention":
+        B, T, H, D, dtype, bias = kw["B"], kw["T"], kw["H"], kw["D"], kw["dtype"], kw["bias"]
+        hs = 2  # two heads of one batch element: T*T*2 fp32 scores at a time
+        q, k, v, do = (torch.randn(1, T, hs, D, generator=g).to(dtype) for _ in range(4))
+        bs = None if bias is None else bias[:1, :hs if bias.shape[1] > 1 else 1].cpu()
+
+        def run():
+            oracle.attention_fwd(q, k, v, bs)
+            oracle.attention_bwd(do, q, k, v, bs)
+        t = _cpu_time(run, reps=1)
+        flops = 14.0 * hs * T * T * D
+        return {"value": round(flops / t / 1e12, 4), "unit": "TFLOP/s", "ms": round(t * 1e3, 1), "cores": cores, "kind": "port",
+                "sample": f"oracle attention_fwd+attention_bwd on 2 of {B * H} (batch, head) pairs"}
+    raise ValueError(kind)
+
 def spin_up(torch, fn, seconds=0.06):
     """Untimed launches for `seconds`: after an idle spell (allocation, input generation on the host) the GPU
     needs tens of milliseconds of work before its clocks reach their steady state, and a kernel timed during
@@ -185,7 +243,7 @@ def time_api(torch, fn, iters=30, warmup=5):
     return a.elapsed_time(b) / iters
 
 
-def attention_case(torch, name, B, T, H, D, dtype, bias_kind, iters=20):
+def attention_case(torch, name, B, T, H, D, dtype, bias_kind, iters=20, with_cpu=False):
     """fwd+bwd through the C ABI with events around the forward and the backward call"""
     from rgd_triton_amd import _hip
 
@@ -250,7 +308,8 @@ def attention_case(torch, name, B, T, H, D, dtype, bias_kind, iters=20):
     tot = f_ms + b_ms
     # every bias element is read by the forward, the dQ and the dK/dV kernel, once per head it applies to
     bias_gbs = None if bias is None else round(3.0 * B * H * T * T * bias.element_size() / tot / 1e6, 1)
-    return {"workload": name, "bias_read_gbs": bias_gbs, "fwd_ms": round(f_ms, 4), "bwd_ms": round(b_ms, 4),
+    cpu = cpu_extra(torch, "attention", B=B, T=T, H=H, D=D, dtype=dtype, bias=bias) if with_cpu else None
+    return {"workload": name, "cpu_baseline": cpu, "bias_read_gbs": bias_gbs, "fwd_ms": round(f_ms, 4), "bwd_ms": round(b_ms, 4),
             "tflops": round(flops / tot / 1e9, 2), "fwd_tflops": round(flops * 4 / 14 / f_ms / 1e9, 2),
             "bwd_tflops": round(flops * 10 / 14 / b_ms / 1e9, 2), "frac_mfma_peak": round(flops / tot / 1e9 / MFMA_PEAK_TFLOPS, 4)}
 
@@ -291,7 +350,7 @@ def rows_result(torch, name, fwd, bwd, fwd_bytes, bwd_bytes, nsets, api=None):
     return r
 
 
-def rms_case(torch, name, B, shapes, dtype, nsets, with_api=True):
+def rms_case(torch, name, B, shapes, dtype, nsets, with_api=True, with_cpu=False):
     """FusedRMSNorm (one shape) or FusedRMSNorm2 (two shapes) forward+backward, shared (C,) weights"""
     import rgd_triton_amd as rgd
     from rgd_triton_amd import _hip
@@ -338,10 +397,12 @@ def rms_case(torch, name, B, shapes, dtype, nsets, with_api=True):
             xb = x2[0].clone().requires_grad_(True)
             m = rgd.FusedRMSNorm2((C1, C2), device="cuda", dtype=dtype)
             api = lambda: torch.autograd.grad(m(xa, xb), (xa, xb, m.weight1, m.weight2), (d1[0], d2[0]))
-    return rows_result(torch, name, fwd, bwd, 2 * n, 3 * n, nsets, api)
+    r = rows_result(torch, name, fwd, bwd, 2 * n, 3 * n, nsets, api)
+    r["cpu_baseline"] = cpu_extra(torch, "rms", B=B, shapes=shapes, dtype=dtype) if with_cpu else None
+    return r
 
 
-def head_ln_case(torch, name, B, T, H, D, dtype, nsets):
+def head_ln_case(torch, name, B, T, H, D, dtype, nsets, with_cpu=False):
     import rgd_triton_amd as rgd
     from rgd_triton_amd import _hip
 
@@ -365,10 +426,12 @@ def head_ln_case(torch, name, B, T, H, D, dtype, nsets):
     m = rgd.FusedHeadLayerNorm()
     api = lambda: torch.autograd.grad(m(qa, ka, heads_second=False), (qa, ka), (gq[0], gk[0]))
     n = 2 * B * T * H * D * torch.empty(0, dtype=dtype).element_size()
-    return rows_result(torch, name, fwd, bwd, 2 * n, 3 * n, nsets, api)
+    r = rows_result(torch, name, fwd, bwd, 2 * n, 3 * n, nsets, api)
+    r["cpu_baseline"] = cpu_extra(torch, "head_ln", B=B, T=T, H=H, D=D, dtype=dtype) if with_cpu else None
+    return r
 
 
-def extras(torch, only=""):
+def extras(torch, only="", with_cpu=False):
     import rgd_triton_amd as rgd
 
     out = []
@@ -378,22 +441,22 @@ def extras(torch, only=""):
         return not only or only == n
 
     if want("attn_c3"):
-        out.append(attention_case(torch, "attn_c3: (4,4096,16,64) bf16 no bias", 4, 4096, 16, 64, bf, None))
+        out.append(attention_case(torch, "attn_c3: (4,4096,16,64) bf16 no bias", 4, 4096, 16, 64, bf, None, with_cpu=with_cpu))
     if want("attn_c4"):
-        out.append(attention_case(torch, "attn_c4: (2,2048,16,128) fp16 full bias", 2, 2048, 16, 128, torch.float16, "full"))
+        out.append(attention_case(torch, "attn_c4: (2,2048,16,128) fp16 full bias", 2, 2048, 16, 128, torch.float16, "full", with_cpu=with_cpu))
     if want("attn_c5"):
-        out.append(attention_case(torch, "attn_c5: (2,4352,24,64) bf16 broadcast bias", 2, 4352, 24, 64, bf, "broadcast"))
+        out.append(attention_case(torch, "attn_c5: (2,4352,24,64) bf16 broadcast bias", 2, 4352, 24, 64, bf, "broadcast", with_cpu=with_cpu))
 
     # buffer sets are sized so that their sum exceeds the 256 MB Infinity Cache
     if want("rms_c1"):
-        out.append(rms_case(torch, "rms_c1: FusedRMSNorm (4,1024,1024) fp32 fwd+bwd", 4, [(1024, 1024)], torch.float32, 12))
+        out.append(rms_case(torch, "rms_c1: FusedRMSNorm (4,1024,1024) fp32 fwd+bwd", 4, [(1024, 1024)], torch.float32, 12, with_cpu=with_cpu))
     if want("rms2_c5"):
         out.append(rms_case(torch, "rms2_c5: FusedRMSNorm2 (2,4096,1536)+(2,256,1536) bf16 fwd+bwd", 2,
-                            [(4096, 1536), (256, 1536)], bf, 12))
+                            [(4096, 1536), (256, 1536)], bf, 12, with_cpu=with_cpu))
     if want("rms_wide"):
         out.append(rms_case(torch, "rms_wide: FusedRMSNorm (8,4096,4096) bf16 fwd+bwd", 8, [(4096, 4096)], bf, 3, with_api=False))
     if want("headln_c5"):
-        out.append(head_ln_case(torch, "headln_c5: FusedHeadLayerNorm q,k (2,4352,24,64) bf16 fwd+bwd", 2, 4352, 24, 64, bf, 6))
+        out.append(head_ln_case(torch, "headln_c5: FusedHeadLayerNorm q,k (2,4352,24,64) bf16 fwd+bwd", 2, 4352, 24, 64, bf, 6, with_cpu=with_cpu))
     return out
 
 
@@ -409,7 +472,7 @@ def main():
     torch.cuda.set_device(0)
 
     if args.only:
-        print(json.dumps({"extra": extras(torch, args.only)}))
+        print(json.dumps({"extra": extras(torch, args.only, with_cpu=not args.skip_cpu)}))
         return
     if args.calib_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").random_()
@@ -456,7 +519,7 @@ def main():
     if not args.skip_extra:
         del sets, fns
         torch.cuda.empty_cache()
-        result["extra"] = extras(torch)
+        result["extra"] = extras(torch, with_cpu=not args.skip_cpu)
     print(json.dumps(result))
 
 
