@@ -74,6 +74,8 @@ template <typename T> __device__ __forceinline__ uint32_t pack2(float lo, float 
     return __builtin_bit_cast(uint32_t, t);
 }
 
+template <int N> struct IntC { static constexpr int value = N; };  // compile-time flag passed by value
+
 // Bias kinds of the kernel templates: no bias, bias stored in the tensor dtype T, bias stored in fp32.
 enum { BIAS_OFF = 0, BIAS_SAME = 1, BIAS_F32 = 2 };
 template <typename T, int BIAS> struct BiasElem { typedef T type; };

@@ -132,11 +132,15 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
     const int voff0 = ld_key0 * (int)p.v.sn + ld_dc0 * 8;
     const bool fast_tiles = vec && p.D == DPAD;  // full rows, 16-byte loads: no masking except in the last tile
     u32x4 kst[LOADS], vst[LOADS];
-    auto issue_loads = [&](int tile) {
+    // FAST (compile time): the caller knows the tile is full and the 16-byte path applies, so the loads are
+    // straight-line code.  The main loop below runs on FAST steps only: with the element-wise loader of ragged
+    // tiles inside the same loop, the compiler has to wait for every outstanding load before a tile's first
+    // matrix instruction (registers shared between the two loaders), and the prefetch hides nothing.
+    auto issue_loads = [&](int tile, auto FAST) {
         const int key0 = tile * ATTN_BN;
         const T* kt = kbase + (int64_t)key0 * p.k.sn;
         const T* vt = vbase + (int64_t)key0 * p.v.sn;
-        if (REGULAR && fast_tiles && key0 + ATTN_BN <= p.Tk) {
+        if (decltype(FAST)::value || (REGULAR && fast_tiles && key0 + ATTN_BN <= p.Tk)) {
 #pragma unroll
             for (int i = 0; i < LOADS; ++i) {
                 // uniform part (tile base + i*ROWS_PER_PASS rows) + fixed per-thread offset
@@ -163,7 +167,7 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
     };
 
     if (t_begin < t_end) {
-        issue_loads(t_begin);
+        issue_loads(t_begin, IntC<0>{});
         store_tiles(t_begin & 1);
     }
     __syncthreads();
@@ -182,14 +186,16 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
             bias_cur.load(bias_row, t_begin * ATTN_BN, g, p.Tk, p.bias_vec && (t_begin + 1) * ATTN_BN <= p.Tk);
     }
 
-    for (int j = t_begin; j < t_end; ++j) {
+    // One key tile.  FAST: tiles j and j+1 are full tiles on the 16-byte path (and the bias, if any, is aligned).
+    auto tile_step = [&](const int j, auto FAST) __attribute__((always_inline)) {
+        constexpr bool F = decltype(FAST)::value != 0;
         const int buf = j & 1;
         const int key0 = j * ATTN_BN;
-        const bool tail = key0 + ATTN_BN > p.Tk;
-        if (j + 1 < t_end) {
-            issue_loads(j + 1);
+        const bool tail = !F && key0 + ATTN_BN > p.Tk;
+        if (F || j + 1 < t_end) {
+            issue_loads(j + 1, FAST);
             if constexpr (HAS_BIAS)
-                bias_nxt.load(bias_row, key0 + ATTN_BN, g, p.Tk, p.bias_vec && key0 + 2 * ATTN_BN <= p.Tk);
+                bias_nxt.load(bias_row, key0 + ATTN_BN, g, p.Tk, F || (p.bias_vec && key0 + 2 * ATTN_BN <= p.Tk));
         }
         if constexpr (!SPLIT_HALVES) {
             // d <= 64: both 32-key halves of the tile go through the softmax together
@@ -376,11 +382,19 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
             }
         }
 
-        if (j + 1 < t_end) {
+        if (F || j + 1 < t_end) {
             store_tiles(buf ^ 1);
             if constexpr (HAS_BIAS) bias_cur = bias_nxt;
         }
         __syncthreads();
+    };
+    {
+        // tiles below n_fast are full and take the 16-byte path; a FAST step also prefetches tile j+1
+        const bool fast_ok = REGULAR && fast_tiles && (!HAS_BIAS || p.bias_vec);
+        const int n_fast = fast_ok ? min(t_end, p.Tk / ATTN_BN) : t_begin;
+        int j = t_begin;
+        for (; j + 1 < n_fast; ++j) tile_step(j, IntC<1>{});
+        for (; j < t_end; ++j) tile_step(j, IntC<0>{});
     }
 
     const float l_tot = l_run + lane_xor32(l_run);
