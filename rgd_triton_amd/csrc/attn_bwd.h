@@ -186,11 +186,14 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
     }
     const bool fast_tiles = vec && p.D == DPAD;
     u32x4 kst[LOADS], vst[LOADS];
-    auto issue_loads = [&](int tile) {
+    // FAST (compile time): the tile is known to be full and on the 16-byte path.  The main loop runs on FAST steps
+    // only; with the element-wise loader of ragged tiles in the same loop the compiler waits for every outstanding
+    // load before a tile's first matrix instruction, and the prefetch hides nothing.
+    auto issue_loads = [&](int tile, auto FAST) {
         const int key0 = tile * BN;
         const T* kt = kbase + (int64_t)key0 * p.k.sn;
         const T* vt = vbase + (int64_t)key0 * p.v.sn;
-        if (fast_tiles && key0 + BN <= p.Tk) {
+        if (decltype(FAST)::value || (fast_tiles && key0 + BN <= p.Tk)) {
 #pragma unroll
             for (int i = 0; i < LOADS; ++i) {
                 kst[i] = *reinterpret_cast<const u32x4*>(kt + koff[i]);
@@ -213,7 +216,7 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
         }
     };
     if (t_begin < t_end) {
-        issue_loads(t_begin);
+        issue_loads(t_begin, IntC<0>{});
         store_tiles(t_begin & 1);
     }
     __syncthreads();
@@ -227,13 +230,16 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
         if (t_begin < t_end) bias_cur.load(bias_row, t_begin * BN, g, p.Tk, p.bias_vec && (t_begin + 1) * BN <= p.Tk);
     }
 
-    for (int j = t_begin; j < t_end; ++j) {
+    // One key tile.  FAST: tiles j and j+1 are full tiles on the 16-byte path (and the bias, if any, is aligned).
+    auto tile_step = [&](const int j, auto FAST) __attribute__((always_inline)) {
+        constexpr bool F = decltype(FAST)::value != 0;
         const int buf = j & 1;
         const int key0 = j * BN;
-        const bool tail = key0 + BN > p.Tk;
-        if (j + 1 < t_end) {
-            issue_loads(j + 1);
-            if constexpr (HAS_BIAS) bias_nxt.load(bias_row, key0 + BN, g, p.Tk, p.bias_vec && key0 + 2 * BN <= p.Tk);
+        const bool tail = !F && key0 + BN > p.Tk;
+        if (F || j + 1 < t_end) {
+            issue_loads(j + 1, FAST);
+            if constexpr (HAS_BIAS)
+                bias_nxt.load(bias_row, key0 + BN, g, p.Tk, F || (p.bias_vec && key0 + 2 * BN <= p.Tk));
         }
         float bias_v[NKB][16];
         if constexpr (HAS_BIAS) bias_cur.decode(bias_v);
@@ -307,11 +313,19 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
                 acc[d] = MM::run(as_v8<T>(a), bop, acc[d]);
             }
         }
-        if (j + 1 < t_end) {
+        if (F || j + 1 < t_end) {
             store_tiles(buf ^ 1);
             if constexpr (HAS_BIAS) bias_cur = bias_nxt;
         }
         __syncthreads();
+    };
+    {
+        // tiles below n_fast are full and take the 16-byte path; a FAST step also prefetches tile j+1
+        const bool fast_ok = fast_tiles && (!HAS_BIAS || p.bias_vec);
+        const int n_fast = fast_ok ? min(t_end, p.Tk / BN) : t_begin;
+        int j = t_begin;
+        for (; j + 1 < n_fast; ++j) tile_step(j, IntC<1>{});
+        for (; j < t_end; ++j) tile_step(j, IntC<0>{});
     }
 
     if (item.nparts > 1) {  // part of a split item: leave the unscaled fp32 sums
@@ -460,12 +474,16 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_D
     }
     const bool fast_tiles = vec && p.D == DPAD;
     u32x4 qst[LOADS], dst[LOADS];
-    float lse_st = 0.f, delta_st = 0.f;
-    auto issue_loads = [&](int tile) {
+    float lse_st = 0.f, delta_st = 0.f;  // raw values as loaded; they are transformed when they are stored to LDS
+    bool row_st = false;                 // the row exists
+    // FAST (compile time): all BQ query rows of the tile exist and the 16-byte path applies.  The main loop runs on
+    // FAST steps only (see the dQ kernel).
+    auto issue_loads = [&](int tile, auto FAST) {
+        constexpr bool F = decltype(FAST)::value != 0;
         const int q0 = tile * BQ;
         const T* qt = qbase + (int64_t)q0 * p.q.sn;
         const T* dot = dobase + (int64_t)q0 * p.dout.sn;
-        if (fast_tiles && q0 + BQ <= p.Tq) {
+        if (F || (fast_tiles && q0 + BQ <= p.Tq)) {
 #pragma unroll
             for (int i = 0; i < LOADS; ++i) {
                 if (TASKS % BWD_THREADS == 0 || tid + i * BWD_THREADS < TASKS) {
@@ -483,11 +501,11 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_D
         }
         if (tid < BQ) {
             const int q = q0 + tid;
-            const bool ok = q < p.Tq;
-            const float l = lsep[ok ? q : 0];
-            // rows that do not exist or have no finite logit get probability 0 (exp2(-inf))
-            lse_st = (ok && l != -INFINITY) ? -l * kLog2e : -INFINITY;
-            delta_st = ok ? -deltap[q] : 0.f;  // negated: it is what the dP accumulator starts from
+            const bool ok = F || q < p.Tq;
+            // only the loads here: using the values now would make the wavefront wait for every load issued above
+            lse_st = lsep[ok ? q : 0];
+            delta_st = deltap[ok ? q : 0];
+            row_st = ok;
         }
     };
     auto store_tiles = [&](int buf) {
@@ -502,12 +520,14 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_D
             }
         }
         if (tid < BQ) {
-            st[tid] = lse_st;
-            st[BQ + tid] = delta_st;
+            // rows that do not exist or have no finite logit get probability 0 (exp2(-inf)); delta is stored negated:
+            // it is what the dP accumulator starts from
+            st[tid] = (row_st && lse_st != -INFINITY) ? -lse_st * kLog2e : -INFINITY;
+            st[BQ + tid] = row_st ? -delta_st : 0.f;
         }
     };
     if (tile_begin < ntiles) {
-        issue_loads(tile_begin);
+        issue_loads(tile_begin, IntC<0>{});
         store_tiles(tile_begin & 1);
     }
     __syncthreads();
@@ -519,26 +539,28 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_D
     const TB* bias_base = nullptr;  // bias of this batch and head (wavefront-uniform)
     uint32_t bias_lane_off = 0;     // this lane's key column, 16*g rows down
     BiasColumn<TB> bias_cur[NSUB], bias_nxt[NSUB];  // fetched one tile ahead of use
-    auto bias_load = [&](BiasColumn<TB> (&dst)[NSUB], int tile) {
+    auto bias_load = [&](BiasColumn<TB> (&dst)[NSUB], int tile, auto FAST) {
 #pragma unroll
         for (int u = 0; u < NSUB; ++u) {
             const int q0 = tile * BQ + u * 32;
             // the ragged sub-tile clamps rows per lane half: its row base is that of the lane's own first row
             dst[u].load(bias_base + (int64_t)q0 * p.bias.sn, p.bias.sn, bias_lane_off, q0 + g * 16, p.Tq,
-                        q0 + 32 <= p.Tq);
+                        decltype(FAST)::value != 0 || q0 + 32 <= p.Tq);
         }
     };
     if constexpr (HAS_BIAS) {
         bias_base = static_cast<const TB*>(p.bias.ptr) + b * p.bias.sb + h * p.bias.sh;
         bias_lane_off = (uint32_t)k_ld + (uint32_t)(g * 16) * (uint32_t)p.bias.sn;
-        if (tile_begin < ntiles) bias_load(bias_cur, tile_begin);
+        if (tile_begin < ntiles) bias_load(bias_cur, tile_begin, IntC<0>{});
     }
 
-    for (int j = tile_begin; j < ntiles; ++j) {
+    // One tile of BQ query rows.  FAST: tile j+1 is a full tile on the 16-byte path.
+    auto tile_step = [&](const int j, auto FAST) __attribute__((always_inline)) {
+        constexpr bool F = decltype(FAST)::value != 0;
         const int buf = j & 1;
-        if (j + 1 < ntiles) {
-            issue_loads(j + 1);
-            if constexpr (HAS_BIAS) bias_load(bias_nxt, j + 1);
+        if (F || j + 1 < ntiles) {
+            issue_loads(j + 1, FAST);
+            if constexpr (HAS_BIAS) bias_load(bias_nxt, j + 1, FAST);
         }
         const T* qs = reinterpret_cast<const T*>(smem_raw + buf * BUFB);
         const T* dos = qs + TILE;
@@ -623,7 +645,7 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_D
                 }
             }
         }
-        if (j + 1 < ntiles) {
+        if (F || j + 1 < ntiles) {
             store_tiles(buf ^ 1);
             if constexpr (HAS_BIAS) {
 #pragma unroll
@@ -631,6 +653,13 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_D
             }
         }
         __syncthreads();
+    };
+    {
+        // tiles below n_fast have all their query rows and take the 16-byte path; a FAST step prefetches tile j+1
+        const int n_fast = fast_tiles ? min(ntiles, p.Tq / BQ) : tile_begin;
+        int j = tile_begin;
+        for (; j + 1 < n_fast; ++j) tile_step(j, IntC<1>{});
+        for (; j < ntiles; ++j) tile_step(j, IntC<0>{});
     }
 
     if (item.nparts > 1) {  // part of a split item: leave the unscaled fp32 sums, dK then dV
