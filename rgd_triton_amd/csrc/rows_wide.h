@@ -12,6 +12,9 @@
 // independent of scheduling.  (Combining the rows inside the first kernel, with arrival tickets, was
 // measured slower: every level of such a tree costs several microseconds of cross-XCD round trips.)
 #pragma once
+#ifndef RGD_WIDE_RMS_FWD_64
+#define RGD_WIDE_RMS_FWD_64 1
+#endif
 
 #include "common.h"
 

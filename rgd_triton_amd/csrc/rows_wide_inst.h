@@ -11,7 +11,7 @@ static int wide_launch_one(const WideParams& p, dim3 grid, size_t lds, hipStream
     constexpr int U = wide_unroll(BWD, NV, VEC);
     constexpr int NW = wide_waves(OP, BWD);
     // the host never selects more elements per lane than this (they would not stay in registers)
-    if constexpr (NV * VEC <= (OP == WIDE_RMS ? 32 : 64)) {
+    if constexpr (NV * VEC <= ((OP == WIDE_RMS && (BWD || !RGD_WIDE_RMS_FWD_64)) ? 32 : 64)) {
         hipLaunchKernelGGL((wide_rows_kernel<T, OP, BWD, G, NV, VEC, VECTOR, U, NW, WPR>), grid, dim3(NW * 64), lds, s,
                            p);
         return 0;
