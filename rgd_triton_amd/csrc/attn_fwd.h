@@ -20,6 +20,9 @@
 // rare after the first tiles.  p = exp2(t) <= 256 is safe for fp16/bf16 operands and fp32 sums, and
 // LSE = (m + log2(l)) * ln2 does not depend on where m sits.
 #pragma once
+#ifndef RGD_FWD_LAZY_MAX
+#define RGD_FWD_LAZY_MAX 1
+#endif
 
 #include "attn_common.h"
 
@@ -27,6 +30,7 @@ constexpr int ATTN_BM = 128;  // query rows per workgroup
 constexpr int ATTN_BN = 64;   // keys per tile
 constexpr int ATTN_THREADS = 256;
 constexpr float ATTN_RESCALE_THRESHOLD = 8.0f;  // log2 units
+constexpr float ATTN_LAZY_LIMIT = 16384.0f;     // partial row sum of one tile above which the maximum is looked at
 
 struct AttnFwdParams {
     AttnTensor q, k, v, bias, o;
@@ -218,7 +222,6 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
 
             // ---- t = logit - m_ref (log2 domain) ----
             const float m_off = m_ref == -INFINITY ? 0.f : m_ref;
-            float tmax = -INFINITY;
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb) {
                 if constexpr (HAS_BIAS) {
@@ -232,51 +235,80 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
                 }
             }
             const bool diag = p.causal && (key0 + ATTN_BN - 1 > qb * ATTN_BM + wave * 32);
-            if (tail || diag) {
+            // running maximum of the tile and, if needed, a move of the reference exponent (first finite logit of
+            // the row, or growth > 2^8): rescales the accumulators and shifts the logits
+            auto max_and_move = [&]() __attribute__((always_inline)) {
+                float tmax = -INFINITY;
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int key = key0 + kb * 32 + g * 16 + v;
-                        if (key >= p.Tk || (p.causal && key > q_row)) s[kb][v] = -INFINITY;
-                    }
-            }
+                    for (int v = 0; v < 16; v += 2) tmax = fmaxf(fmaxf(tmax, s[kb][v]), s[kb][v + 1]);
+                tmax = fmaxf(tmax, lane_xor32(tmax));
+                const bool move = (m_ref == -INFINITY) ? (tmax != -INFINITY) : (tmax > ATTN_RESCALE_THRESHOLD);
+                if (__builtin_amdgcn_ballot_w64(move) != 0) {
+                    const float m_old = m_ref == -INFINITY ? 0.f : m_ref;
+                    const float shift = move ? tmax : 0.f;
+                    const float alpha = move ? __builtin_amdgcn_exp2f(m_ref - (m_old + shift)) : 1.f;  // 0 when m_ref was -inf
+                    m_ref = move ? m_old + shift : m_ref;
+                    l_run *= alpha;
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+                    for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                for (int v = 0; v < 16; v += 2) tmax = fmaxf(fmaxf(tmax, s[kb][v]), s[kb][v + 1]);
-            tmax = fmaxf(tmax, lane_xor32(tmax));
-
-            // move the reference exponent only when needed (first finite logit of the row, or growth > 2^8)
-            const bool move = (m_ref == -INFINITY) ? (tmax != -INFINITY) : (tmax > ATTN_RESCALE_THRESHOLD);
-            if (__builtin_amdgcn_ballot_w64(move) != 0) {
-                const float shift = move ? tmax : 0.f;
-                const float alpha = move ? __builtin_amdgcn_exp2f(m_ref - (m_off + shift)) : 1.f;  // 0 when m_ref was -inf
-                m_ref = move ? m_off + shift : m_ref;
-                l_run *= alpha;
+                        for (int v = 0; v < 16; ++v) s[kb][v] -= shift;
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
+                    for (int d = 0; d < NDB; ++d)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) s[kb][v] -= shift;
-#pragma unroll
-                for (int d = 0; d < NDB; ++d)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) oacc[d][v] *= alpha;
-            }
-
-            // ---- p = exp2(t), packed to the operand type ----
-            uint32_t pk[2][8];
-            float lsum0 = 0.f, lsum1 = 0.f;  // the row sum uses the unrounded fp32 values: LSE keeps fp32 accuracy
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int v = 0; v < 16; v += 2) {
-                    const float p0 = __builtin_amdgcn_exp2f(s[kb][v]);
-                    const float p1 = __builtin_amdgcn_exp2f(s[kb][v + 1]);
-                    pk[kb][v / 2] = pack2<T>(p0, p1);
-                    lsum0 += p0;
-                    lsum1 += p1;
+                        for (int v = 0; v < 16; ++v) oacc[d][v] *= alpha;
                 }
+            };
+            // p = exp2(t), packed to the operand type; the row sum uses the unrounded fp32 values (LSE keeps fp32
+            // accuracy)
+            uint32_t pk[2][8];
+            float lsum0 = 0.f, lsum1 = 0.f;
+            auto exp_pack = [&]() __attribute__((always_inline)) {
+                lsum0 = 0.f;
+                lsum1 = 0.f;
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int v = 0; v < 16; v += 2) {
+                        const float p0 = __builtin_amdgcn_exp2f(s[kb][v]);
+                        const float p1 = __builtin_amdgcn_exp2f(s[kb][v + 1]);
+                        pk[kb][v / 2] = pack2<T>(p0, p1);
+                        lsum0 += p0;
+                        lsum1 += p1;
+                    }
+            };
+            bool done = false;
+#if RGD_FWD_LAZY_MAX
+            if constexpr (F) {
+                // Full tile away from the causal diagonal: exponentiate against the current reference first and
+                // look at the maximum only if that went wrong somewhere in the wavefront (row without a reference
+                // yet, or a partial row sum beyond 2^14, i.e. some p that large: still far inside fp16/bf16 range).
+                if (!diag) {
+                    exp_pack();
+                    const bool bad = (m_ref == -INFINITY) || !(lsum0 + lsum1 <= ATTN_LAZY_LIMIT);  // catches inf and NaN
+                    if (__builtin_amdgcn_ballot_w64(bad) != 0) {
+                        max_and_move();
+                        exp_pack();
+                    }
+                    done = true;
+                }
+            }
+#endif
+            if (!done) {
+                if (tail || diag) {
+#pragma unroll
+                    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            const int key = key0 + kb * 32 + g * 16 + v;
+                            if (key >= p.Tk || (p.causal && key > q_row)) s[kb][v] = -INFINITY;
+                        }
+                }
+                max_and_move();
+                exp_pack();
+            }
             l_run += lsum0 + lsum1;
 
             // ---- O^T += V^T . P^T ----
