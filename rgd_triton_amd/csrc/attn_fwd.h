@@ -132,8 +132,18 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
     const int ld_key0 = tid / CPR, ld_dc0 = tid % CPR;
     auto chunk_key = [&](int i) { return REGULAR ? ld_key0 + i * ROWS_PER_PASS : (tid + i * ATTN_THREADS) / CPR; };
     auto chunk_dc = [&](int i) { return REGULAR ? ld_dc0 : (tid + i * ATTN_THREADS) % CPR; };
+    // element offsets of this thread's chunks inside a tile: one offset plus a uniform row step (REGULAR), or one
+    // offset per chunk (head dim 96)
     const int koff0 = ld_key0 * (int)p.k.sn + ld_dc0 * 8;
     const int voff0 = ld_key0 * (int)p.v.sn + ld_dc0 * 8;
+    int koff[REGULAR ? 1 : LOADS], voff[REGULAR ? 1 : LOADS];
+    if constexpr (!REGULAR) {
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) {
+            koff[i] = chunk_key(i) * (int)p.k.sn + chunk_dc(i) * 8;
+            voff[i] = chunk_key(i) * (int)p.v.sn + chunk_dc(i) * 8;
+        }
+    }
     const bool fast_tiles = vec && p.D == DPAD;  // full rows, 16-byte loads: no masking except in the last tile
     u32x4 kst[LOADS], vst[LOADS];
     // FAST (compile time): the caller knows the tile is full and the 16-byte path applies, so the loads are
@@ -144,12 +154,16 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
         const int key0 = tile * ATTN_BN;
         const T* kt = kbase + (int64_t)key0 * p.k.sn;
         const T* vt = vbase + (int64_t)key0 * p.v.sn;
-        if (decltype(FAST)::value || (REGULAR && fast_tiles && key0 + ATTN_BN <= p.Tk)) {
+        if (decltype(FAST)::value || (fast_tiles && key0 + ATTN_BN <= p.Tk)) {
 #pragma unroll
-            for (int i = 0; i < LOADS; ++i) {
-                // uniform part (tile base + i*ROWS_PER_PASS rows) + fixed per-thread offset
-                kst[i] = *reinterpret_cast<const u32x4*>(kt + (int64_t)(i * ROWS_PER_PASS) * p.k.sn + koff0);
-                vst[i] = *reinterpret_cast<const u32x4*>(vt + (int64_t)(i * ROWS_PER_PASS) * p.v.sn + voff0);
+            for (int i = 0; i < LOADS; ++i) {  // wavefront-uniform tile base + fixed per-thread offset
+                if constexpr (REGULAR) {
+                    kst[i] = *reinterpret_cast<const u32x4*>(kt + (int64_t)(i * ROWS_PER_PASS) * p.k.sn + koff0);
+                    vst[i] = *reinterpret_cast<const u32x4*>(vt + (int64_t)(i * ROWS_PER_PASS) * p.v.sn + voff0);
+                } else {
+                    kst[i] = *reinterpret_cast<const u32x4*>(kt + koff[i]);
+                    vst[i] = *reinterpret_cast<const u32x4*>(vt + voff[i]);
+                }
             }
         } else {
 #pragma unroll
@@ -422,7 +436,7 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
     };
     {
         // tiles below n_fast are full and take the 16-byte path; a FAST step also prefetches tile j+1
-        const bool fast_ok = REGULAR && fast_tiles && (!HAS_BIAS || p.bias_vec);
+        const bool fast_ok = fast_tiles && (!HAS_BIAS || p.bias_vec);
         const int n_fast = fast_ok ? min(t_end, p.Tk / ATTN_BN) : t_begin;
         int j = t_begin;
         for (; j + 1 < n_fast; ++j) tile_step(j, IntC<1>{});
