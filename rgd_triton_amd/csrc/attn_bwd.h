@@ -174,17 +174,23 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
 
     const T* kbase = static_cast<const T*>(p.k.ptr) + b * p.k.sb + h * p.k.sh;
     const T* vbase = static_cast<const T*>(p.v.ptr) + b * p.v.sb + h * p.v.sh;
+    // A head dim below the padded one (40, 80, 112, ...) leaves whole chunks past the end of a row: the fast loader
+    // reads chunk 0 of the row in their place and store_tiles writes zeros (pad_mask bit i = chunk i).
+    const bool padded = p.D != DPAD;
+    uint32_t pad_mask = 0;
     int ld_key[LOADS], ld_dc[LOADS], koff[LOADS], voff[LOADS], soff[LOADS];
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
         const int id = tid + i * BWD_THREADS;
         ld_key[i] = id / CPR;
         ld_dc[i] = id % CPR;
-        koff[i] = ld_key[i] * (int)p.k.sn + ld_dc[i] * 8;
-        voff[i] = ld_key[i] * (int)p.v.sn + ld_dc[i] * 8;
+        const bool pad = ld_dc[i] * 8 >= p.D;
+        pad_mask |= (pad ? 1u : 0u) << i;
+        koff[i] = ld_key[i] * (int)p.k.sn + (pad ? 0 : ld_dc[i] * 8);
+        voff[i] = ld_key[i] * (int)p.v.sn + (pad ? 0 : ld_dc[i] * 8);
         soff[i] = ld_key[i] * ST + ld_dc[i] * 8;
     }
-    const bool fast_tiles = vec && p.D == DPAD;
+    const bool fast_tiles = vec;  // rows made of whole 16-byte chunks
     u32x4 kst[LOADS], vst[LOADS];
     // FAST (compile time): the tile is known to be full and on the 16-byte path.  The main loop runs on FAST steps
     // only; with the element-wise loader of ragged tiles in the same loop the compiler waits for every outstanding
@@ -209,6 +215,11 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
         }
     };
     auto store_tiles = [&](int buf) {
+        if (padded) {
+#pragma unroll
+            for (int i = 0; i < LOADS; ++i)
+                if (pad_mask >> i & 1u) kst[i] = vst[i] = u32x4{0u, 0u, 0u, 0u};
+        }
 #pragma unroll
         for (int i = 0; i < LOADS; ++i) {
             *reinterpret_cast<u32x4*>(ks_base + buf * TILE + soff[i]) = kst[i];
@@ -462,17 +473,22 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_D
     const int tile_begin = tile_first + (int)((int64_t)(ntiles_all - tile_first) * item.part / item.nparts);
     const int ntiles = tile_first + (int)((int64_t)(ntiles_all - tile_first) * (item.part + 1) / item.nparts);
 
+    // chunks past the end of a row (head dim below the padded one): as in the dQ kernel
+    const bool padded = p.D != DPAD;
+    uint32_t pad_mask = 0;
     int ld_row[LOADS], ld_dc[LOADS], qoff[LOADS], dooff[LOADS], soff[LOADS];
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
         const int id = tid + i * BWD_THREADS;
         ld_row[i] = id / CPR;
         ld_dc[i] = id % CPR;
-        qoff[i] = ld_row[i] * (int)p.q.sn + ld_dc[i] * 8;
-        dooff[i] = ld_row[i] * (int)p.dout.sn + ld_dc[i] * 8;
+        const bool pad = ld_dc[i] * 8 >= p.D;
+        pad_mask |= (pad ? 1u : 0u) << i;
+        qoff[i] = ld_row[i] * (int)p.q.sn + (pad ? 0 : ld_dc[i] * 8);
+        dooff[i] = ld_row[i] * (int)p.dout.sn + (pad ? 0 : ld_dc[i] * 8);
         soff[i] = ld_row[i] * ST + ld_dc[i] * 8;
     }
-    const bool fast_tiles = vec && p.D == DPAD;
+    const bool fast_tiles = vec;  // rows made of whole 16-byte chunks
     u32x4 qst[LOADS], dst[LOADS];
     float lse_st = 0.f, delta_st = 0.f;  // raw values as loaded; they are transformed when they are stored to LDS
     bool row_st = false;                 // the row exists
@@ -512,6 +528,11 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_D
         T* qs = reinterpret_cast<T*>(smem_raw + buf * BUFB);
         T* ds = qs + TILE;
         float* st = reinterpret_cast<float*>(smem_raw + buf * BUFB + 2 * TILE * 2);
+        if (padded) {
+#pragma unroll
+            for (int i = 0; i < LOADS; ++i)
+                if (pad_mask >> i & 1u) qst[i] = dst[i] = u32x4{0u, 0u, 0u, 0u};
+        }
 #pragma unroll
         for (int i = 0; i < LOADS; ++i) {
             if (TASKS % BWD_THREADS == 0 || tid + i * BWD_THREADS < TASKS) {

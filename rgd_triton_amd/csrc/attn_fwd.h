@@ -134,17 +134,23 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
     auto chunk_dc = [&](int i) { return REGULAR ? ld_dc0 : (tid + i * ATTN_THREADS) % CPR; };
     // element offsets of this thread's chunks inside a tile: one offset plus a uniform row step (REGULAR), or one
     // offset per chunk (head dim 96)
-    const int koff0 = ld_key0 * (int)p.k.sn + ld_dc0 * 8;
-    const int voff0 = ld_key0 * (int)p.v.sn + ld_dc0 * 8;
+    // A head dim below the padded one (40, 80, 112, ...) leaves whole chunks past the end of a row: the fast
+    // loader reads chunk 0 of the row in their place and store_tiles writes zeros.
+    const bool padded = p.D != DPAD;
+    auto chunk_pad = [&](int i) { return chunk_dc(i) * 8 >= p.D; };  // recomputed where used: no register held
+    auto chunk_col = [&](int i) { return chunk_pad(i) ? 0 : chunk_dc(i) * 8; };
+    const int koff0 = ld_key0 * (int)p.k.sn + chunk_col(0);
+    const int voff0 = ld_key0 * (int)p.v.sn + chunk_col(0);
     int koff[REGULAR ? 1 : LOADS], voff[REGULAR ? 1 : LOADS];
     if constexpr (!REGULAR) {
 #pragma unroll
         for (int i = 0; i < LOADS; ++i) {
-            koff[i] = chunk_key(i) * (int)p.k.sn + chunk_dc(i) * 8;
-            voff[i] = chunk_key(i) * (int)p.v.sn + chunk_dc(i) * 8;
+            koff[i] = chunk_key(i) * (int)p.k.sn + chunk_col(i);
+            voff[i] = chunk_key(i) * (int)p.v.sn + chunk_col(i);
         }
     }
-    const bool fast_tiles = vec && p.D == DPAD;  // full rows, 16-byte loads: no masking except in the last tile
+    // rows made of whole 16-byte chunks: straight-line loads, no masking except in the last tile
+    const bool fast_tiles = vec && p.D % 8 == 0;
     u32x4 kst[LOADS], vst[LOADS];
     // FAST (compile time): the caller knows the tile is full and the 16-byte path applies, so the loads are
     // straight-line code.  The main loop below runs on FAST steps only: with the element-wise loader of ragged
@@ -176,6 +182,11 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
         }
     };
     auto store_tiles = [&](int buf) {
+        if (padded) {
+#pragma unroll
+            for (int i = 0; i < LOADS; ++i)
+                if (chunk_pad(i)) kst[i] = vst[i] = u32x4{0u, 0u, 0u, 0u};
+        }
 #pragma unroll
         for (int i = 0; i < LOADS; ++i) {
             const int so = chunk_key(i) * ST + chunk_dc(i) * 8;

@@ -107,6 +107,32 @@ def test_flash_attn_head_dims(Tq, Tk, d, dtype):
 
 @pytest.mark.parametrize("dtype", HALF)
 @pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("bias_type", ["none", "cube"])
+@pytest.mark.parametrize("d", [40, 80, 112])
+def test_flash_attn_padded_head_dim_long(d, bias_type, causal, dtype):
+    """head dims made of whole 16-byte chunks but below the kernels' padded width, over enough tiles for the main
+    loop; q/k/v/do are column slices of wider tensors whose other columns hold NaN, so a read past the end of a
+    row (into the neighbouring columns) would show up in every output"""
+    g = gen(7)
+    B, H, Tq, Tk = 1, 2, 448, 520
+    wide = lambda T: torch.full((B, T, H, d + 24), float("nan"), dtype=dtype)
+    q, k, v, do = wide(Tq), wide(Tk), wide(Tk), wide(Tq)
+    for t, T in ((q, Tq), (k, Tk), (v, Tk), (do, Tq)):
+        t[..., 8:8 + d] = randn(g, B, T, H, d, dtype=dtype)
+    qs, ks, vs, dos = (t[..., 8:8 + d] for t in (q, k, v, do))
+    bias = make_bias(g, bias_type, B, H, Tq, Tk, dtype)
+    from rgd_triton_amd import flash_attn_func
+
+    qg, kg, vg, dog = (t.cuda()[..., 8:8 + d] for t in (q, k, v, do))
+    qg.requires_grad_(True), kg.requires_grad_(True), vg.requires_grad_(True)
+    o, lse = flash_attn_func(qg, kg, vg, None if bias is None else bias.cuda(), causal, None, return_lse=True)
+    dq, dk, dv = torch.autograd.grad(o, (qg, kg, vg), dog)
+    qc, kc, vc, doc = (t.contiguous() for t in (qs, ks, vs, dos))
+    check((o, lse, dq, dk, dv), reference(qc, kc, vc, bias, doc, causal), Tq, grad_mult=3, name=f"d={d}")
+
+
+@pytest.mark.parametrize("dtype", HALF)
+@pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("bias_type", ["none", "vector", "cube"])
 @pytest.mark.parametrize("Tq,Tk", [(128, 128), (200, 200), (113, 203), (300, 150), (1, 64)])
 def test_flash_attn_causal_vector_fp32bias(Tq, Tk, bias_type, causal, dtype):
