@@ -355,6 +355,10 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
 // ------------------------------------------------------------------------------------------------
 // dK / dV kernel
 // ------------------------------------------------------------------------------------------------
+// 1: LDS operand reads of the dK/dV kernel run one step ahead of the matrix instructions (head dims above 64)
+#ifndef RGD_DKV_READ_AHEAD
+#define RGD_DKV_READ_AHEAD 1
+#endif
 #ifndef RGD_DKV_OCC
 #define RGD_DKV_OCC 2  // wavefronts per SIMD of the dK/dV kernel without bias at head dims <= 64
 #endif
@@ -600,15 +604,42 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_D
                     dp[u][4 * i + e] = c[e];
                 }
             }
+        // The operand reads run one step ahead of the matrix instructions that use them (the scheduling barriers keep
+        // them there).  Left alone, the compiler issues each read right before its use, and with one wavefront per
+        // SIMD (head dims above 64) nothing else covers the LDS round trip.  With two wavefronts it makes no difference.
+        constexpr bool READ_AHEAD = RGD_DKV_READ_AHEAD && DPAD > 64;
+        if constexpr (READ_AHEAD) {
+            u32x4 qa[2][NSUB], da[2][NSUB];
+            auto read_step = [&](int c) __attribute__((always_inline)) {
 #pragma unroll
-        for (int c = 0; c < NC; ++c)
+                for (int u = 0; u < NSUB; ++u) {
+                    qa[c & 1][u] = *reinterpret_cast<const u32x4*>(qs + u * 32 * ST + a_off + c * 16);
+                    da[c & 1][u] = *reinterpret_cast<const u32x4*>(dos + u * 32 * ST + a_off + c * 16);
+                }
+            };
+            read_step(0);
 #pragma unroll
-            for (int u = 0; u < NSUB; ++u) {
-                const u32x4 qa = *reinterpret_cast<const u32x4*>(qs + u * 32 * ST + a_off + c * 16);
-                s[u] = MM::run(as_v8<T>(qa), kreg[c], s[u]);
-                const u32x4 da = *reinterpret_cast<const u32x4*>(dos + u * 32 * ST + a_off + c * 16);
-                dp[u] = MM::run(as_v8<T>(da), vreg[c], dp[u]);
+            for (int c = 0; c < NC; ++c) {
+                if (c + 1 < NC) read_step(c + 1);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int u = 0; u < NSUB; ++u) {
+                    s[u] = MM::run(as_v8<T>(qa[c & 1][u]), kreg[c], s[u]);
+                    dp[u] = MM::run(as_v8<T>(da[c & 1][u]), vreg[c], dp[u]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
+        } else {
+#pragma unroll
+            for (int c = 0; c < NC; ++c)
+#pragma unroll
+                for (int u = 0; u < NSUB; ++u) {
+                    const u32x4 qa = *reinterpret_cast<const u32x4*>(qs + u * 32 * ST + a_off + c * 16);
+                    s[u] = MM::run(as_v8<T>(qa), kreg[c], s[u]);
+                    const u32x4 da = *reinterpret_cast<const u32x4*>(dos + u * 32 * ST + a_off + c * 16);
+                    dp[u] = MM::run(as_v8<T>(da), vreg[c], dp[u]);
+                }
+        }
 #pragma unroll
         for (int u = 0; u < NSUB; ++u) {
             const int q0 = j * BQ + u * 32;
@@ -646,23 +677,50 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_D
                 dsk[v / 2] = pack2<T>(p0 * dp[u][v], p1 * dp[u][v + 1]);
             }
             // dV^T += dO^T . P ;  dK^T += Q^T . dS
-#pragma unroll
-            for (int jj = 0; jj < 2; ++jj) {
-                const u32x4 praw = {pk[jj * 4 + 0], pk[jj * 4 + 1], pk[jj * 4 + 2], pk[jj * 4 + 3]};
-                const u32x4 draw = {dsk[jj * 4 + 0], dsk[jj * 4 + 1], dsk[jj * 4 + 2], dsk[jj * 4 + 3]};
-                const typename MM::V8 pb = as_v8<T>(praw), db = as_v8<T>(draw);
-#pragma unroll
-                for (int d = 0; d < NDB; ++d) {
+            if constexpr (READ_AHEAD) {
+                u32x4 dta[2], qta[2];  // transposed dO and Q operands, one (jj, d) step ahead
+                auto read_t = [&](int t) __attribute__((always_inline)) {
+                    const int jj = t / NDB, d = t % NDB;
                     const T* dsrc = dos + u * 32 * ST + tr_off + jj * 8 * ST + d * 32;
                     const u32x2 dlo = lds_read_tr<T>(dsrc);
                     const u32x2 dhi = lds_read_tr<T>(dsrc + 4 * ST);
-                    const u32x4 da = {dlo[0], dlo[1], dhi[0], dhi[1]};
-                    dv_acc[d] = MM::run(as_v8<T>(da), pb, dv_acc[d]);
+                    dta[t & 1] = u32x4{dlo[0], dlo[1], dhi[0], dhi[1]};
                     const T* qsrc = qs + u * 32 * ST + tr_off + jj * 8 * ST + d * 32;
                     const u32x2 qlo = lds_read_tr<T>(qsrc);
                     const u32x2 qhi = lds_read_tr<T>(qsrc + 4 * ST);
-                    const u32x4 qa = {qlo[0], qlo[1], qhi[0], qhi[1]};
-                    dk_acc[d] = MM::run(as_v8<T>(qa), db, dk_acc[d]);
+                    qta[t & 1] = u32x4{qlo[0], qlo[1], qhi[0], qhi[1]};
+                };
+                read_t(0);
+#pragma unroll
+                for (int t = 0; t < 2 * NDB; ++t) {
+                    const int jj = t / NDB, d = t % NDB;
+                    if (t + 1 < 2 * NDB) read_t(t + 1);
+                    __builtin_amdgcn_sched_barrier(0);
+                    const u32x4 praw = {pk[jj * 4 + 0], pk[jj * 4 + 1], pk[jj * 4 + 2], pk[jj * 4 + 3]};
+                    const u32x4 draw = {dsk[jj * 4 + 0], dsk[jj * 4 + 1], dsk[jj * 4 + 2], dsk[jj * 4 + 3]};
+                    dv_acc[d] = MM::run(as_v8<T>(dta[t & 1]), as_v8<T>(praw), dv_acc[d]);
+                    dk_acc[d] = MM::run(as_v8<T>(qta[t & 1]), as_v8<T>(draw), dk_acc[d]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else {
+#pragma unroll
+                for (int jj = 0; jj < 2; ++jj) {
+                    const u32x4 praw = {pk[jj * 4 + 0], pk[jj * 4 + 1], pk[jj * 4 + 2], pk[jj * 4 + 3]};
+                    const u32x4 draw = {dsk[jj * 4 + 0], dsk[jj * 4 + 1], dsk[jj * 4 + 2], dsk[jj * 4 + 3]};
+                    const typename MM::V8 pb = as_v8<T>(praw), db = as_v8<T>(draw);
+#pragma unroll
+                    for (int d = 0; d < NDB; ++d) {
+                        const T* dsrc = dos + u * 32 * ST + tr_off + jj * 8 * ST + d * 32;
+                        const u32x2 dlo = lds_read_tr<T>(dsrc);
+                        const u32x2 dhi = lds_read_tr<T>(dsrc + 4 * ST);
+                        const u32x4 da = {dlo[0], dlo[1], dhi[0], dhi[1]};
+                        dv_acc[d] = MM::run(as_v8<T>(da), pb, dv_acc[d]);
+                        const T* qsrc = qs + u * 32 * ST + tr_off + jj * 8 * ST + d * 32;
+                        const u32x2 qlo = lds_read_tr<T>(qsrc);
+                        const u32x2 qhi = lds_read_tr<T>(qsrc + 4 * ST);
+                        const u32x4 qa = {qlo[0], qlo[1], qhi[0], qhi[1]};
+                        dk_acc[d] = MM::run(as_v8<T>(qa), db, dk_acc[d]);
+                    }
                 }
             }
         }
