@@ -580,8 +580,11 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_D
     }
 
     // One tile of BQ query rows.  FAST: tile j+1 is a full tile on the 16-byte path.
-    auto tile_step = [&](const int j, auto FAST) __attribute__((always_inline)) {
+    // NOMASK: every key of the workgroup exists and the launch is not causal, so no logit is masked (and the step
+    // is one basic block for the instruction scheduler).
+    auto tile_step = [&](const int j, auto FAST, auto NOMASK) __attribute__((always_inline)) {
         constexpr bool F = decltype(FAST)::value != 0;
+        constexpr bool NM = decltype(NOMASK)::value != 0;
         const int buf = j & 1;
         if (F || j + 1 < ntiles) {
             issue_loads(j + 1, FAST);
@@ -660,12 +663,14 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_D
 #pragma unroll
                 for (int v = 0; v < 16; ++v) s[u][v] = fmaf(s[u][v], p.scale_log2, nlse[v]);
             }
-            const bool diag = p.causal && (q0 < kblk * BWD_BM + wave * 32 + 32);
-            if (!k_valid || diag) {
+            if constexpr (!NM) {
+                const bool diag = p.causal && (q0 < kblk * BWD_BM + wave * 32 + 32);
+                if (!k_valid || diag) {
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int q = q0 + g * 16 + v;
-                    if (!k_valid || key > q) s[u][v] = -INFINITY;
+                    for (int v = 0; v < 16; ++v) {
+                        const int q = q0 + g * 16 + v;
+                        if (!k_valid || key > q) s[u][v] = -INFINITY;
+                    }
                 }
             }
             uint32_t pk[8], dsk[8];
@@ -737,8 +742,12 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_D
         // tiles below n_fast have all their query rows and take the 16-byte path; a FAST step prefetches tile j+1
         const int n_fast = fast_tiles ? min(ntiles, p.Tq / BQ) : tile_begin;
         int j = tile_begin;
-        for (; j + 1 < n_fast; ++j) tile_step(j, IntC<1>{});
-        for (; j < ntiles; ++j) tile_step(j, IntC<0>{});
+        if (!p.causal && (kblk + 1) * BWD_BM <= p.Tk) {
+            for (; j + 1 < n_fast; ++j) tile_step(j, IntC<1>{}, IntC<1>{});
+        } else {
+            for (; j + 1 < n_fast; ++j) tile_step(j, IntC<1>{}, IntC<0>{});
+        }
+        for (; j < ntiles; ++j) tile_step(j, IntC<0>{}, IntC<0>{});
     }
 
     if (item.nparts > 1) {  // part of a split item: leave the unscaled fp32 sums, dK then dV
