@@ -94,7 +94,7 @@ int wide_launch(const char* name, int op, bool bwd, int64_t B, const WideHalfArg
     for (const WideHalfArgs* a : as) {
         RGD_REQUIRE(a->T >= 0 && a->T < (1ll << 31) && a->C >= 0 && a->C < (1ll << 31), RGD_ERR_INVALID,
                     "%s: shape out of range", name);
-        if (a->T == 0 || a->C == 0) continue;
+        if (B == 0 || a->T == 0 || a->C == 0) continue;  // nothing to do for this tensor (its pointers may be null)
         RGD_REQUIRE(a->x && a->x->ptr && a->y && a->y->ptr, RGD_ERR_INVALID, "%s: null tensor", name);
         RGD_REQUIRE(!bwd || (a->dy && a->dy->ptr), RGD_ERR_INVALID, "%s: null gradient", name);
         RGD_REQUIRE(!has_w || (a->w && a->w->ptr && rgd_dtype_ok(a->w_dtype)), RGD_ERR_INVALID, "%s: bad weight", name);

@@ -119,7 +119,7 @@ class RMS_Func(torch.autograd.Function):
         _seen(ctx.kernel_cache, "bwd_dw", _sig(w))
         dx = torch.empty_like(x)
         dw = torch.empty(w.shape, dtype=w.dtype, device=w.device)
-        if T == 0:
+        if B * T == 0:
             dw.zero_()
             return dx, dw, None, None
         wbuf, wsz = _rms_scratch(x, None)
@@ -170,9 +170,9 @@ class Fused_RMS_Func(torch.autograd.Function):
         dx1, dx2 = torch.empty_like(x1), torch.empty_like(x2)
         dw1 = torch.empty(w1.shape, dtype=w1.dtype, device=w1.device)
         dw2 = torch.empty(w2.shape, dtype=w2.dtype, device=w2.device)
-        if T1 == 0:
+        if B * T1 == 0:
             dw1.zero_()
-        if T2 == 0:
+        if B * T2 == 0:
             dw2.zero_()
         wbuf, wsz = _rms_scratch(x1, x2)
         lib = _hip.lib()
