@@ -24,8 +24,21 @@ def randn(g, *shape, dtype=torch.float32, scale=1.0, shift=0.0):
     return (torch.randn(*shape, generator=g, dtype=torch.float32) * scale + shift).to(dtype)
 
 
+def dev(t):
+    """t on the GPU with the same sizes, strides and storage offset.  `t.to("cuda")` makes a view with gaps
+    contiguous, which would take the strided and unaligned layouts out of a test; here the whole underlying buffer
+    is rebuilt on the GPU, NaN outside the view, so a read beyond the view shows up in the result."""
+    if t.is_contiguous() or 0 in t.stride() or not t.is_floating_point():
+        return t.to(DEV)
+    n = t.untyped_storage().nbytes() // t.element_size()
+    base = torch.full((n,), float("nan"), dtype=t.dtype, device=DEV)
+    v = base.as_strided(t.size(), t.stride(), t.storage_offset())
+    v.copy_(t)
+    return v
+
+
 def to_gpu(*ts, requires_grad=False):
-    out = [t.to(DEV).detach().requires_grad_(requires_grad) for t in ts]
+    out = [dev(t).detach().requires_grad_(requires_grad) for t in ts]
     return out if len(out) > 1 else out[0]
 
 

@@ -8,7 +8,7 @@ import random
 import pytest
 import torch
 
-from helpers import assert_close, assert_close_allow_inf, gen, oracle, randn, to_gpu
+from helpers import assert_close, assert_close_allow_inf, dev, gen, oracle, randn, to_gpu
 from test_flash_attn import check, reference
 
 pytestmark = pytest.mark.gpu
@@ -61,9 +61,9 @@ def test_random_attention(seed):
         dead = torch.randperm(Tk, generator=g)[: Tk // 3]
         dead = dead[dead != 0]  # with a causal mask the first query row sees key 0 only: keep it, so that no row
         bias[..., dead] = float("-inf")  # is fully masked (the PyTorch reference gives NaN there, the kernels 0)
-    qg, kg, vg = (t.to("cuda").detach().requires_grad_(True) for t in (q, k, v))
+    qg, kg, vg = to_gpu(q, k, v, requires_grad=True)
     o, lse = flash_attn_func(qg, kg, vg, None if bias is None else bias.to("cuda"), causal, None, return_lse=True)
-    dq, dk, dv = torch.autograd.grad(o, (qg, kg, vg), do.to("cuda"))
+    dq, dk, dv = torch.autograd.grad(o, (qg, kg, vg), dev(do))
     ref = reference(q, k, v, bias, do, causal)
     if bias is not None and bias.dtype != dtype:  # the low-precision comparison run adds the bias in q's dtype
         ref = ref[:3] + reference(q, k, v, bias.to(dtype), do, causal)[3:]
@@ -96,7 +96,7 @@ def test_random_wide_rows(seed):
         if op == "rms":
             xg, wg = to_gpu(x1, w1, requires_grad=True)
             y = triton_rms_func_fn(xg, wg, 1e-6)
-            dx, dw = torch.autograd.grad(y, (xg, wg), d1.to("cuda"))
+            dx, dw = torch.autograd.grad(y, (xg, wg), dev(d1))
             dx_r, dw_r = oracle.rms_bwd(d1, x1, w1, 1e-6)
             assert_close(y, oracle.rms_fwd(x1, w1, 1e-6), dtype, "rms", name + " y")
             assert_close(dx, dx_r, dtype, "rms", name + " dx")
@@ -104,7 +104,7 @@ def test_random_wide_rows(seed):
         else:
             a, b_, wa, wb = to_gpu(x1, x2, w1, w2, requires_grad=True)
             y1, y2 = triton_fused_rms_func_fn(a, b_, wa, wb, 1e-6)
-            ga = torch.autograd.grad((y1, y2), (a, b_, wa, wb), (d1.to("cuda"), d2.to("cuda")))
+            ga = torch.autograd.grad((y1, y2), (a, b_, wa, wb), (dev(d1), dev(d2)))
             r1, r2 = oracle.rms_bwd(d1, x1, w1, 1e-6), oracle.rms_bwd(d2, x2, w2, 1e-6)
             assert_close(y1, oracle.rms_fwd(x1, w1, 1e-6), dtype, "rms", name + " y1")
             assert_close(y2, oracle.rms_fwd(x2, w2, 1e-6), dtype, "rms", name + " y2")
@@ -115,13 +115,13 @@ def test_random_wide_rows(seed):
     elif op == "l2":
         xg = to_gpu(x1, requires_grad=True)
         y = triton_norm_func_fn(xg, 1e-6)
-        (dx,) = torch.autograd.grad(y, xg, d1.to("cuda"))
+        (dx,) = torch.autograd.grad(y, xg, dev(d1))
         assert_close(y, oracle.l2_fwd(x1, 1e-6), dtype, name=name + " y")
         assert_close_allow_inf(dx, oracle.l2_bwd(d1, x1, 1e-6), dtype, name=name + " dx")
     else:
         a, b_ = to_gpu(x1, x2, requires_grad=True)
         y1, y2 = triton_fused_norm_func_fn(a, b_, 1e-6)
-        ga = torch.autograd.grad((y1, y2), (a, b_), (d1.to("cuda"), d2.to("cuda")))
+        ga = torch.autograd.grad((y1, y2), (a, b_), (dev(d1), dev(d2)))
         assert_close(y1, oracle.l2_fwd(x1, 1e-6), dtype, name=name + " y1")
         assert_close(y2, oracle.l2_fwd(x2, 1e-6), dtype, name=name + " y2")
         assert_close_allow_inf(ga[0], oracle.l2_bwd(d1, x1, 1e-6), dtype, name=name + " dx1")
@@ -147,7 +147,7 @@ def test_random_head_ops(seed):
     qg, kg = to_gpu(q, k, requires_grad=True)
     if op == "ln":
         qo, ko = triton_fused_ln_func_fn(qg, kg, heads_second, 1e-6)
-        dq, dk = torch.autograd.grad((qo, ko), (qg, kg), (gq.to("cuda"), gk.to("cuda")))
+        dq, dk = torch.autograd.grad((qo, ko), (qg, kg), (dev(gq), dev(gk)))
         for a, r, n in ((qo, oracle.head_ln_fwd(q), "qo"), (ko, oracle.head_ln_fwd(k), "ko"),
                         (dq, oracle.head_ln_bwd(gq, q), "dq"), (dk, oracle.head_ln_bwd(gk, k), "dk")):
             assert_close(a, r, dtype, name=f"{name} {n}")
@@ -167,6 +167,6 @@ def test_random_head_ops(seed):
         ref_f = oracle.ln_rope_fwd(q, k, pe, cutoff, heads_second, 1e-6)
         ref_b = oracle.ln_rope_bwd(gq, gk, q, k, pe, cutoff, heads_second, 1e-6)
         tol = "ln_rope"
-    dq, dk = torch.autograd.grad((qo, ko), (qg, kg), (gq.to("cuda"), gk.to("cuda")))
+    dq, dk = torch.autograd.grad((qo, ko), (qg, kg), (dev(gq), dev(gk)))
     for a, r, n in ((qo, ref_f[0], "qo"), (ko, ref_f[1], "ko"), (dq, ref_b[0], "dq"), (dk, ref_b[1], "dk")):
         assert_close(a, r, dtype, tol, f"{name} {n}")
