@@ -582,13 +582,19 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_D
     // One tile of BQ query rows.  FAST: tile j+1 is a full tile on the 16-byte path.
     // NOMASK: every key of the workgroup exists and the launch is not causal, so no logit is masked (and the step
     // is one basic block for the instruction scheduler).
-    auto tile_step = [&](const int j, auto FAST, auto NOMASK) __attribute__((always_inline)) {
+    // PING 0 / 1: one half of a pair of steps that swap the roles of the two bias register sets (0 uses bias_cur and
+    // fills bias_nxt, 1 the other way round), so no step copies 16 registers per sub-tile; 2: a single step that
+    // uses bias_cur and copies bias_nxt into it at its end.
+    auto tile_step = [&](const int j, auto FAST, auto NOMASK, auto PING) __attribute__((always_inline)) {
         constexpr bool F = decltype(FAST)::value != 0;
         constexpr bool NM = decltype(NOMASK)::value != 0;
+        constexpr int PP = decltype(PING)::value;
+        BiasColumn<TB>(&b_use)[NSUB] = pick_ref<PP == 1>(bias_cur, bias_nxt);
+        BiasColumn<TB>(&b_fill)[NSUB] = pick_ref<PP == 1>(bias_nxt, bias_cur);
         const int buf = j & 1;
         if (F || j + 1 < ntiles) {
             issue_loads(j + 1, FAST);
-            if constexpr (HAS_BIAS) bias_load(bias_nxt, j + 1, FAST);
+            if constexpr (HAS_BIAS) bias_load(b_fill, j + 1, FAST);
         }
         const T* qs = reinterpret_cast<const T*>(smem_raw + buf * BUFB);
         const T* dos = qs + TILE;
@@ -656,7 +662,7 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_D
             }
             if constexpr (HAS_BIAS) {
                 float bias_r[16];
-                bias_cur[u].decode(bias_r);
+                b_use[u].decode(bias_r);
 #pragma unroll
                 for (int v = 0; v < 16; ++v) s[u][v] = fmaf(s[u][v], p.scale_log2, fmaf(bias_r[v], kLog2e, nlse[v]));
             } else {
@@ -731,7 +737,7 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_D
         }
         if (F || j + 1 < ntiles) {
             store_tiles(buf ^ 1);
-            if constexpr (HAS_BIAS) {
+            if constexpr (HAS_BIAS && PP == 2) {
 #pragma unroll
                 for (int u = 0; u < NSUB; ++u) bias_cur[u] = bias_nxt[u];
             }
@@ -743,11 +749,17 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_D
         const int n_fast = fast_tiles ? min(ntiles, p.Tq / BQ) : tile_begin;
         int j = tile_begin;
         if (!p.causal && (kblk + 1) * BWD_BM <= p.Tk) {
-            for (; j + 1 < n_fast; ++j) tile_step(j, IntC<1>{}, IntC<1>{});
+            if constexpr (HAS_BIAS) {
+                for (; j + 2 < n_fast; j += 2) {
+                    tile_step(j, IntC<1>{}, IntC<1>{}, IntC<0>{});
+                    tile_step(j + 1, IntC<1>{}, IntC<1>{}, IntC<1>{});
+                }
+            }
+            for (; j + 1 < n_fast; ++j) tile_step(j, IntC<1>{}, IntC<1>{}, IntC<2>{});
         } else {
-            for (; j + 1 < n_fast; ++j) tile_step(j, IntC<1>{}, IntC<0>{});
+            for (; j + 1 < n_fast; ++j) tile_step(j, IntC<1>{}, IntC<0>{}, IntC<2>{});
         }
-        for (; j < ntiles; ++j) tile_step(j, IntC<0>{}, IntC<0>{});
+        for (; j < ntiles; ++j) tile_step(j, IntC<0>{}, IntC<0>{}, IntC<2>{});
     }
 
     if (item.nparts > 1) {  // part of a split item: leave the unscaled fp32 sums, dK then dV

@@ -74,7 +74,13 @@ template <typename T> __device__ __forceinline__ uint32_t pack2(float lo, float 
     return __builtin_bit_cast(uint32_t, t);
 }
 
-template <int N> struct IntC { static constexpr int value = N; };  // compile-time flag passed by value
+template <int N> struct IntC { static constexpr int value = N; };
+
+// first or second of two references, chosen at compile time
+template <bool SECOND, typename X> __device__ __forceinline__ X& pick_ref(X& a, X& b) {
+    if constexpr (SECOND) return b;
+    else return a;
+}  // compile-time flag passed by value
 
 // Bias kinds of the kernel templates: no bias, bias stored in the tensor dtype T, bias stored in fp32.
 enum { BIAS_OFF = 0, BIAS_SAME = 1, BIAS_F32 = 2 };
