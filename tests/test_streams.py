@@ -45,3 +45,37 @@ def test_two_streams_match_default_stream():
         for got in outs:
             for a, r in zip(got, ref):
                 assert torch.equal(a, r)
+
+
+def test_two_host_threads():
+    """two host threads, each on its own stream, call the operators at the same time (autograd adds its own worker
+    thread for the backward passes): results equal the single-threaded ones bit for bit"""
+    import threading
+
+    pa, pb = _problem(3, 257, 768, 200, 2, 64), _problem(4, 129, 2048, 333, 3, 32)
+    ref = {"a": _run(pa), "b": _run(pb)}
+    torch.cuda.synchronize()
+    outs, errors = {"a": [], "b": []}, []
+
+    def work(name, prob):
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for _ in range(8):
+                    outs[name].append(_run(prob))
+            stream.synchronize()
+        except Exception as e:  # surfaced in the main thread below
+            errors.append((name, repr(e)))
+
+    threads = [threading.Thread(target=work, args=("a", pa)), threading.Thread(target=work, args=("b", pb))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
+    for name in ("a", "b"):
+        assert len(outs[name]) == 8
+        for got in outs[name]:
+            for a, r in zip(got, ref[name]):
+                assert torch.equal(a, r)
