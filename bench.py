@@ -309,9 +309,36 @@ def attention_case(torch, name, B, T, H, D, dtype, bias_kind, iters=20, with_cpu
     # every bias element is read by the forward, the dQ and the dK/dV kernel, once per head it applies to
     bias_gbs = None if bias is None else round(3.0 * B * H * T * T * bias.element_size() / tot / 1e6, 1)
     cpu = cpu_extra(torch, "attention", B=B, T=T, H=H, D=D, dtype=dtype, bias=bias) if with_cpu else None
-    return {"workload": name, "cpu_baseline": cpu, "bias_read_gbs": bias_gbs, "fwd_ms": round(f_ms, 4), "bwd_ms": round(b_ms, 4),
+    sdpa = torch_sdpa_case(torch, q, k, v, do, bias, flops) if with_cpu else None
+    return {"workload": name, "cpu_baseline": cpu, "torch_sdpa": sdpa, "bias_read_gbs": bias_gbs, "fwd_ms": round(f_ms, 4), "bwd_ms": round(b_ms, 4),
             "tflops": round(flops / tot / 1e9, 2), "fwd_tflops": round(flops * 4 / 14 / f_ms / 1e9, 2),
             "bwd_tflops": round(flops * 10 / 14 / b_ms / 1e9, 2), "frac_mfma_peak": round(flops / tot / 1e9 / MFMA_PEAK_TFLOPS, 4)}
+
+
+def torch_sdpa_case(torch, q, k, v, do, bias, flops, iters=10):
+    """PyTorch's own fused attention (scaled_dot_product_attention, whatever backend it picks on this GPU) on the same
+    tensors, forward + backward through autograd: a second reported baseline next to the CPU one, not a target."""
+    import torch.nn.functional as F
+
+    try:
+        ql, kl, vl = (t.detach().transpose(1, 2).requires_grad_(True) for t in (q, k, v))  # (B,h,T,d) views
+        dot = do.transpose(1, 2)
+
+        def step(_=None):
+            o = F.scaled_dot_product_attention(ql, kl, vl, attn_mask=bias)
+            torch.autograd.grad(o, (ql, kl, vl), dot)
+
+        spin_up(torch, step, 0.05)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            step()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / iters
+        return {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 2), "what": f"torch {torch.__version__} F.scaled_dot_product_attention fwd+bwd, default backend"}
+    except Exception as e:  # no kernel for this shape / dtype on this build
+        return {"error": f"{type(e).__name__}: {str(e)[:100]}"}
 
 
 def time_pair(torch, fwd, bwd, nsets, iters=60, warmup=8):
