@@ -155,6 +155,47 @@ def cpu_baseline_ln_rope(torch, B=8, T=2048, H=16, D=64, R=32, reps=3):
             "host_cpus": os.cpu_count()}
 
 
+def torch_eager_ln_rope(torch, B=8, T=2048, H=16, D=64, R=32, iters=20):
+    """The headline step written with PyTorch's own GPU operators (F.layer_norm in fp32, the rotation as slices and a
+    stack, autograd for the backward) on the same shapes: what a user has on this GPU without fused kernels.  A second
+    reported baseline, not a target."""
+    import torch.nn.functional as F
+
+    try:
+        g = torch.Generator().manual_seed(1002)
+        q, k, gq, gk = (torch.randn(B, T, H, D, generator=g).to(torch.bfloat16).cuda() for _ in range(4))
+        q.requires_grad_(True)
+        k.requires_grad_(True)
+        inv = 10000.0 ** (-torch.arange(0, R, 2, dtype=torch.float32) / R)
+        ang = torch.arange(T, dtype=torch.float32)[:, None] * inv[None, :]
+        sin = ang.sin().repeat_interleave(2, dim=-1)[None, :, None, :].cuda()
+        cos = ang.cos().repeat_interleave(2, dim=-1)[None, :, None, :].cuda()
+
+        def one(x):
+            y = F.layer_norm(x.float(), (D,), eps=1e-5)
+            r, rest = y[..., :R], y[..., R:]
+            rot = torch.stack((-r[..., 1::2], r[..., 0::2]), dim=-1).flatten(-2)
+            return torch.cat((r * cos + rot * sin, rest), dim=-1).to(x.dtype)
+
+        def step(_=None):
+            qo, ko = one(q), one(k)
+            torch.autograd.grad((qo, ko), (q, k), (gq, gk))
+
+        spin_up(torch, step, 0.05)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            step()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / iters
+        nbytes = 5 * 2 * B * T * H * D * 2
+        return {"value": round(nbytes / ms / 1e6, 1), "unit": "GB/s", "ms_per_step": round(ms, 4),
+                "what": f"torch {torch.__version__} eager operators + autograd on the same GPU, same algorithmic bytes"}
+    except Exception as e:
+        return {"error": f"{type(e).__name__}: {str(e)[:100]}"}
+
+
 # ------------------------------------------------------------------------------------------------
 # extra workloads (reported under "extra", not the headline value)
 # ------------------------------------------------------------------------------------------------
@@ -546,6 +587,9 @@ def main():
     if not args.skip_extra:
         del sets, fns
         torch.cuda.empty_cache()
+        if not args.skip_cpu:
+            result["torch_eager_gpu"] = torch_eager_ln_rope(torch)
+            torch.cuda.empty_cache()
         result["extra"] = extras(torch, with_cpu=not args.skip_cpu)
     print(json.dumps(result))
 
