@@ -127,7 +127,7 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 31, g = lane >> 5;
     const BwdItem item = bwd_item(p);
     const int bid = item.bid;
-    const int qb = bid % p.nblk;
+    const int qb = p.causal ? p.nblk - 1 - bid % p.nblk : bid % p.nblk;  // causal: longest row blocks first
     const int bh = bid / p.nblk;
     const int b = bh / p.H, h = bh - b * p.H;
     const int q_row = qb * BWD_BM + wave * 32 + li;

@@ -89,7 +89,9 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
         part = part_id % p.split_s;
         nparts = p.split_s;
     }
-    const int qb = bid % p.nqb;
+    // causal: the last row blocks of a (batch, head) have the most key tiles; they go first, so that the launch
+    // does not end on its longest workgroups
+    const int qb = p.causal ? p.nqb - 1 - bid % p.nqb : bid % p.nqb;
     const int bh = bid / p.nqb;
     const int b = bh / p.H;
     const int h = bh - b * p.H;
