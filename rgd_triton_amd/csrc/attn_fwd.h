@@ -20,6 +20,10 @@
 // rare after the first tiles.  p = exp2(t) <= 256 is safe for fp16/bf16 operands and fp32 sums, and
 // LSE = (m + log2(l)) * ln2 does not depend on where m sits.
 #pragma once
+// 1: the main loop of the forward without bias (d <= 64) fetches two tiles ahead
+#ifndef RGD_FWD_PREFETCH2
+#define RGD_FWD_PREFETCH2 1
+#endif
 #ifndef RGD_FWD_LAZY_MAX
 #define RGD_FWD_LAZY_MAX 1
 #endif
@@ -153,12 +157,16 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
     }
     // rows made of whole 16-byte chunks: straight-line loads, no masking except in the last tile
     const bool fast_tiles = vec && p.D % 8 == 0;
-    u32x4 kst[LOADS], vst[LOADS];
+    // two staging register sets when the main loop fetches two tiles ahead (PF2), else one
+    constexpr bool PF2 = RGD_FWD_PREFETCH2 && DPAD <= 64 && !HAS_BIAS;
+    u32x4 kst_[PF2 ? 2 : 1][LOADS], vst_[PF2 ? 2 : 1][LOADS];
     // FAST (compile time): the caller knows the tile is full and the 16-byte path applies, so the loads are
     // straight-line code.  The main loop below runs on FAST steps only: with the element-wise loader of ragged
     // tiles inside the same loop, the compiler has to wait for every outstanding load before a tile's first
     // matrix instruction (registers shared between the two loaders), and the prefetch hides nothing.
-    auto issue_loads = [&](int tile, auto FAST) {
+    auto issue_loads = [&](int tile, auto FAST, auto SET) {
+        u32x4(&kst)[LOADS] = kst_[PF2 ? decltype(SET)::value : 0];
+        u32x4(&vst)[LOADS] = vst_[PF2 ? decltype(SET)::value : 0];
         const int key0 = tile * ATTN_BN;
         const T* kt = kbase + (int64_t)key0 * p.k.sn;
         const T* vt = vbase + (int64_t)key0 * p.v.sn;
@@ -183,7 +191,9 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
             }
         }
     };
-    auto store_tiles = [&](int buf) {
+    auto store_tiles = [&](int buf, auto SET) {
+        u32x4(&kst)[LOADS] = kst_[PF2 ? decltype(SET)::value : 0];
+        u32x4(&vst)[LOADS] = vst_[PF2 ? decltype(SET)::value : 0];
         if (padded) {
 #pragma unroll
             for (int i = 0; i < LOADS; ++i)
@@ -198,8 +208,8 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
     };
 
     if (t_begin < t_end) {
-        issue_loads(t_begin, IntC<0>{});
-        store_tiles(t_begin & 1);
+        issue_loads(t_begin, IntC<0>{}, IntC<0>{});
+        store_tiles(t_begin & 1, IntC<0>{});
     }
     __syncthreads();
 
@@ -218,13 +228,18 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
     }
 
     // One key tile.  FAST: tiles j and j+1 are full tiles on the 16-byte path (and the bias, if any, is aligned).
-    auto tile_step = [&](const int j, auto FAST) __attribute__((always_inline)) {
+    // AHEAD 0: the step fetches tile j+1 and stores it at its end.  AHEAD 1 / 2 (j even / odd): it fetches tile j+2
+    // into the staging set of j's parity and stores tile j+1, fetched by the step before, from the other set: the
+    // store no longer waits for loads issued a step ago at most.
+    auto tile_step = [&](const int j, auto FAST, auto AHEAD) __attribute__((always_inline)) {
         constexpr bool F = decltype(FAST)::value != 0;
+        constexpr int AH = decltype(AHEAD)::value;
         const int buf = j & 1;
         const int key0 = j * ATTN_BN;
         const bool tail = !F && key0 + ATTN_BN > p.Tk;
         if (F || j + 1 < t_end) {
-            issue_loads(j + 1, FAST);
+            if constexpr (AH == 0) issue_loads(j + 1, FAST, IntC<0>{});
+            else issue_loads(j + 2, FAST, IntC<AH - 1>{});
             if constexpr (HAS_BIAS)
                 bias_nxt.load(bias_row, key0 + ATTN_BN, g, p.Tk, F || (p.bias_vec && key0 + 2 * ATTN_BN <= p.Tk));
         }
@@ -442,7 +457,7 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
         }
 
         if (F || j + 1 < t_end) {
-            store_tiles(buf ^ 1);
+            store_tiles(buf ^ 1, IntC<(AH == 0 ? 0 : 2 - AH)>{});
             if constexpr (HAS_BIAS) bias_cur = bias_nxt;
         }
         __syncthreads();
@@ -452,8 +467,25 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
         const bool fast_ok = fast_tiles && (!HAS_BIAS || p.bias_vec);
         const int n_fast = fast_ok ? min(t_end, p.Tk / ATTN_BN) : t_begin;
         int j = t_begin;
-        for (; j + 1 < n_fast; ++j) tile_step(j, IntC<1>{});
-        for (; j < t_end; ++j) tile_step(j, IntC<0>{});
+        if constexpr (PF2) {
+            if (n_fast - j >= 4) {
+                // tile j is in LDS; tile j+1 goes into flight here, each step then fetches two tiles ahead
+                if (j & 1) {
+                    issue_loads(j + 1, IntC<1>{}, IntC<0>{});
+                    tile_step(j, IntC<1>{}, IntC<2>{});
+                    ++j;
+                } else {
+                    issue_loads(j + 1, IntC<1>{}, IntC<1>{});
+                }
+                for (; j + 3 < n_fast; j += 2) {
+                    tile_step(j, IntC<1>{}, IntC<1>{});
+                    tile_step(j + 1, IntC<1>{}, IntC<2>{});
+                }
+                // tile j is in LDS and tile j+1 in flight (set of its parity); the steps below fetch it again
+            }
+        }
+        for (; j + 1 < n_fast; ++j) tile_step(j, IntC<1>{}, IntC<0>{});
+        for (; j < t_end; ++j) tile_step(j, IntC<0>{}, IntC<0>{});
     }
 
     const float l_tot = l_run + lane_xor32(l_run);
