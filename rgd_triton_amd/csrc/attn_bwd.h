@@ -94,6 +94,10 @@ __device__ __forceinline__ void store_row16(T* row, int col, int D, bool vec, co
 #ifndef RGD_DQ_BN128
 #define RGD_DQ_BN128 32
 #endif
+// 1: the main loop of the dQ kernel without bias (d <= 64) fetches two tiles ahead
+#ifndef RGD_DQ_PREFETCH2
+#define RGD_DQ_PREFETCH2 1
+#endif
 template <int DPAD> struct DqSmem {
     // keys per tile: 32 at d = 128, where the smaller staging and logit registers let two wavefronts share a SIMD
     static constexpr int BN = DPAD == 128 ? RGD_DQ_BN128 : 64;
@@ -191,11 +195,15 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
         soff[i] = ld_key[i] * ST + ld_dc[i] * 8;
     }
     const bool fast_tiles = vec;  // rows made of whole 16-byte chunks
-    u32x4 kst[LOADS], vst[LOADS];
+    // two staging register sets when the main loop fetches two tiles ahead (PF2), else one
+    constexpr bool PF2 = RGD_DQ_PREFETCH2 && DPAD <= 64 && !HAS_BIAS;
+    u32x4 kst_[PF2 ? 2 : 1][LOADS], vst_[PF2 ? 2 : 1][LOADS];
     // FAST (compile time): the tile is known to be full and on the 16-byte path.  The main loop runs on FAST steps
     // only; with the element-wise loader of ragged tiles in the same loop the compiler waits for every outstanding
     // load before a tile's first matrix instruction, and the prefetch hides nothing.
-    auto issue_loads = [&](int tile, auto FAST) {
+    auto issue_loads = [&](int tile, auto FAST, auto SET) {
+        u32x4(&kst)[LOADS] = kst_[PF2 ? decltype(SET)::value : 0];
+        u32x4(&vst)[LOADS] = vst_[PF2 ? decltype(SET)::value : 0];
         const int key0 = tile * BN;
         const T* kt = kbase + (int64_t)key0 * p.k.sn;
         const T* vt = vbase + (int64_t)key0 * p.v.sn;
@@ -214,7 +222,9 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
             }
         }
     };
-    auto store_tiles = [&](int buf) {
+    auto store_tiles = [&](int buf, auto SET) {
+        u32x4(&kst)[LOADS] = kst_[PF2 ? decltype(SET)::value : 0];
+        u32x4(&vst)[LOADS] = vst_[PF2 ? decltype(SET)::value : 0];
         if (padded) {
 #pragma unroll
             for (int i = 0; i < LOADS; ++i)
@@ -227,8 +237,8 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
         }
     };
     if (t_begin < t_end) {
-        issue_loads(t_begin, IntC<0>{});
-        store_tiles(t_begin & 1);
+        issue_loads(t_begin, IntC<0>{}, IntC<0>{});
+        store_tiles(t_begin & 1, IntC<0>{});
     }
     __syncthreads();
 
@@ -242,13 +252,17 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
     }
 
     // One key tile.  FAST: tiles j and j+1 are full tiles on the 16-byte path (and the bias, if any, is aligned).
-    auto tile_step = [&](const int j, auto FAST) __attribute__((always_inline)) {
+    // AHEAD 0: the step fetches tile j+1 and stores it at its end.  AHEAD 1 / 2 (j even / odd): it fetches tile j+2
+    // into the staging set of j's parity and stores tile j+1, fetched by the step before, from the other set.
+    auto tile_step = [&](const int j, auto FAST, auto AHEAD) __attribute__((always_inline)) {
         constexpr bool F = decltype(FAST)::value != 0;
+        constexpr int AH = decltype(AHEAD)::value;
         const int buf = j & 1;
         const int key0 = j * BN;
         const bool tail = !F && key0 + BN > p.Tk;
         if (F || j + 1 < t_end) {
-            issue_loads(j + 1, FAST);
+            if constexpr (AH == 0) issue_loads(j + 1, FAST, IntC<0>{});
+            else issue_loads(j + 2, FAST, IntC<AH - 1>{});
             if constexpr (HAS_BIAS)
                 bias_nxt.load(bias_row, key0 + BN, g, p.Tk, F || (p.bias_vec && key0 + 2 * BN <= p.Tk));
         }
@@ -325,7 +339,7 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
             }
         }
         if (F || j + 1 < t_end) {
-            store_tiles(buf ^ 1);
+            store_tiles(buf ^ 1, IntC<(AH == 0 ? 0 : 2 - AH)>{});
             if constexpr (HAS_BIAS) bias_cur = bias_nxt;
         }
         __syncthreads();
@@ -335,8 +349,25 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
         const bool fast_ok = fast_tiles && (!HAS_BIAS || p.bias_vec);
         const int n_fast = fast_ok ? min(t_end, p.Tk / BN) : t_begin;
         int j = t_begin;
-        for (; j + 1 < n_fast; ++j) tile_step(j, IntC<1>{});
-        for (; j < t_end; ++j) tile_step(j, IntC<0>{});
+        if constexpr (PF2) {
+            if (n_fast - j >= 4) {
+                // tile j is in LDS; tile j+1 goes into flight here, each step then fetches two tiles ahead
+                if (j & 1) {
+                    issue_loads(j + 1, IntC<1>{}, IntC<0>{});
+                    tile_step(j, IntC<1>{}, IntC<2>{});
+                    ++j;
+                } else {
+                    issue_loads(j + 1, IntC<1>{}, IntC<1>{});
+                }
+                for (; j + 3 < n_fast; j += 2) {
+                    tile_step(j, IntC<1>{}, IntC<1>{});
+                    tile_step(j + 1, IntC<1>{}, IntC<2>{});
+                }
+                // tile j is in LDS and tile j+1 in flight; the steps below fetch it again
+            }
+        }
+        for (; j + 1 < n_fast; ++j) tile_step(j, IntC<1>{}, IntC<0>{});
+        for (; j < t_end; ++j) tile_step(j, IntC<0>{}, IntC<0>{});
     }
 
     if (item.nparts > 1) {  // part of a split item: leave the unscaled fp32 sums
