@@ -19,6 +19,9 @@ the closed-form backward functions follow the reference's kernels.  How each one
   ln_rope_fwd / ln_rope_bwd    composition of the two pinned halves + autograd (fp64)
   attention_fwd / attention_bwd  brute-force python loops in fp64 on tiny inputs, torch.softmax /
                                torch.logsumexp, autograd (fp64), bias-broadcast equivalence
+  attention_lowp               in fp64 it equals attention_fwd and the brute-force loops for every bias form,
+                               causal or not, and its autograd gradients equal attention_bwd; in bf16 / fp16 its
+                               error lies in a measured band around the rounding error of the exact result
   rotary_table                 sin^2 + cos^2 = 1, pair duplication, angle(t) = t * theta^(-2i/R)
 
 No function here is "parity unpinned".

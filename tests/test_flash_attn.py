@@ -49,13 +49,26 @@ def maxdiff(a, b):
     return (a.detach().cpu().float() - b.detach().float()).abs().max().item()
 
 
+# Absolute backstop of every comparison, independent of the low-precision error bar: the error against the fp32
+# oracle, in half-ulps of the tensor dtype at the scale of the largest reference element (of 1 for outputs
+# smaller than that).  The kernels round P and dS once to the operand type and accumulate in fp32: 1-4 half-ulps.
+ABS_HALF_ULPS = 12.0
+
+
+def half_ulp(dtype):
+    return 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+
+
 def check(got, ref, Tq, out_mult=2, grad_mult=2, grad_add=0.0, name=""):
     o, lse, dq, dk, dv = got
     o_ref, lse_ref, g_ref, o_pt, g_pt = ref
     assert not torch.isnan(o).any() and not torch.isnan(dq).any() and not torch.isnan(dk).any() and not torch.isnan(dv).any()
     assert maxdiff(o, o_ref) <= out_mult * maxdiff(o_pt, o_ref) + 1e-5, f"{name} o: {maxdiff(o, o_ref)} vs {maxdiff(o_pt, o_ref)}"
+    hu = ABS_HALF_ULPS * half_ulp(o.dtype)
+    assert maxdiff(o, o_ref) <= hu * max(1.0, o_ref.float().abs().max().item()), f"{name} o: absolute error {maxdiff(o, o_ref)}"
     for a, r, pt, n in zip((dq, dk, dv), g_ref, g_pt, ("dq", "dk", "dv")):
         assert maxdiff(a, r) <= grad_mult * maxdiff(pt, r) + grad_add + 1e-5, f"{name} {n}: {maxdiff(a, r)} vs {maxdiff(pt, r)}"
+        assert maxdiff(a, r) <= hu * max(1.0, r.float().abs().max().item()), f"{name} {n}: absolute error {maxdiff(a, r)}"
     fin = torch.isfinite(lse_ref)
     torch.testing.assert_close(lse[..., :Tq].cpu()[fin], lse_ref[fin], rtol=1e-4, atol=1e-4)
     assert torch.all(lse[..., Tq:] == 0)

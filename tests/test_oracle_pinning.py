@@ -11,7 +11,7 @@ import pytest
 import torch
 import torch.nn.functional as F
 
-from helpers import gen, oracle
+from helpers import gen, oracle, randn
 
 F64 = torch.float64
 
@@ -257,6 +257,72 @@ def test_attention_defaults_and_dead_rows():
     assert torch.all(o[0, 1] == 0) and lse[0, 0, 1] == -math.inf and not torch.isnan(o).any()
     dq, dk, dv = oracle.attention_bwd(r64(g, 1, 3, 1, 16), q, k, v, bias, False, None, F64)
     assert not any(torch.isnan(t).any() for t in (dq, dk, dv)) and torch.all(dq[0, 1] == 0)
+
+
+# ------------------------------------------------------------------------------------------ attention_lowp
+# attention_lowp is the error bar of the GPU attention tests (reference tests/test_flash_attn.py:44-62 with
+# upcast=False, reorder_ops=True).  Two pins: in fp64 it is the same function as attention_fwd (a dropped bias, a
+# wrong scale or mask fails), and in 16-bit types its error sits in a band around the rounding error of the
+# result itself (an accidental upcast falls below the band, an extra source of error above it).
+LOWP_BIASES = [None, (1, 1, 7, 9), (2, 1, 7, 9), (1, 3, 7, 9), (2, 3, 7, 9), (2, 3, 1, 9)]
+
+
+@pytest.mark.parametrize("bias_shape", LOWP_BIASES)
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("d", [8, 12])  # 1/sqrt(12) is not a power of two
+def test_attention_lowp_is_attention_fwd_in_fp64(bias_shape, causal, d):
+    g = gen(20)
+    q, k, v = r64(g, 2, 7, 3, d), r64(g, 2, 9, 3, d), r64(g, 2, 9, 3, d)
+    bias = None if bias_shape is None else r64(g, *bias_shape)
+    o_ref, _ = oracle.attention_fwd(q, k, v, bias, causal, None, F64)
+    o_lp = oracle.attention_lowp(q, k, v, bias, causal)
+    assert o_lp.dtype == F64
+    torch.testing.assert_close(o_lp, o_ref, rtol=1e-12, atol=1e-12)
+    o_brute, _ = brute_attention(q, k, v, bias, causal, 1 / math.sqrt(d))
+    torch.testing.assert_close(o_lp, o_brute, rtol=1e-11, atol=1e-12)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_attention_lowp_gradients_in_fp64(causal):
+    """autograd through attention_lowp (what the GPU tests use as the gradient error bar) equals the closed-form
+    backward"""
+    g = gen(21)
+    q, k, v = (r64(g, 2, 7, 3, 12).requires_grad_(True), r64(g, 2, 9, 3, 12).requires_grad_(True),
+               r64(g, 2, 9, 3, 12).requires_grad_(True))
+    bias, do = r64(g, 2, 3, 7, 9), r64(g, 2, 7, 3, 12)
+    ad = torch.autograd.grad(oracle.attention_lowp(q, k, v, bias, causal), (q, k, v), do)
+    got = oracle.attention_bwd(do, q.detach(), k.detach(), v.detach(), bias, causal, None, F64)
+    for a, r in zip(got, ad):
+        torch.testing.assert_close(a, r, rtol=1e-9, atol=1e-12)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(2, 128, 128, 3, 64), (2, 97, 203, 3, 32), (1, 384, 384, 2, 128)])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_attention_lowp_error_band(dtype, shape, with_bias):
+    """N(0,1) inputs, no mask.  Measured over these cases: the output error of the low-precision run is 2.7-6.4
+    times the error of rounding the exact result to the dtype (that ratio is 1 for a run that upcasts), and the
+    gradient errors are 1.0-4.5 half-ulps of the largest gradient element (at most 0.5 for a run that upcasts)."""
+    B, Tq, Tk, H, d = shape
+    g = gen(22)
+    q, k, v, do = (randn(g, B, T, H, d, dtype=dtype) for T in (Tq, Tk, Tk, Tq))
+    bias = randn(g, B, H, Tq, Tk, dtype=dtype) if with_bias else None
+    f = lambda t: None if t is None else t.float()
+    exact, _ = oracle.attention_fwd(f(q), f(k), f(v), f(bias))                # fp32 in, fp32 out
+    rounded, _ = oracle.attention_fwd(q, k, v, bias)                          # fp32 math, one rounding
+    ql, kl, vl = (t.clone().requires_grad_(True) for t in (q, k, v))
+    lowp = oracle.attention_lowp(ql, kl, vl, bias)
+    assert lowp.dtype == dtype
+    err = (lowp.float() - exact).abs().max().item()
+    err_round = (rounded.float() - exact).abs().max().item()
+    assert 2.0 * err_round <= err <= 10.0 * err_round, f"output error {err} vs rounding error {err_round}"
+    half_ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    g_lp = torch.autograd.grad(lowp, (ql, kl, vl), do)
+    g_ref = oracle.attention_bwd(do, q, k, v, bias)
+    for a, r, n in zip(g_lp, g_ref, ("dq", "dk", "dv")):
+        assert a.dtype == dtype
+        rel = ((a.float() - r.float()).abs().max() / r.float().abs().max()).item() / half_ulp
+        assert 0.7 <= rel <= 8.0, f"{n}: error of the low-precision gradient = {rel} half-ulps of its largest element"
 
 
 # ------------------------------------------------------------------------------------------ tolerances
