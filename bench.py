@@ -434,17 +434,15 @@ def rms_case(torch, name, B, shapes, dtype, nsets, with_api=True, with_cpu=False
     w1 = (1 + 0.1 * torch.randn(C1, device="cuda")).to(dtype)
     w2 = (1 + 0.1 * torch.randn(max(C2, 1), device="cuda")).to(dtype)
     dw1, dw2 = torch.empty_like(w1), torch.empty_like(w2)
-    ws, ct = ctypes.c_size_t(), ctypes.c_size_t()
-    assert lib.rgd_rms_bwd_workspace(B, T1, C1, T2, C2, ctypes.byref(ws), ctypes.byref(ct)) == 0
-    wbuf = torch.empty(max(ws.value, 1), dtype=torch.uint8, device="cuda")
-    cbuf = torch.zeros(max(ct.value, 1), dtype=torch.uint8, device="cuda")
+    ws = lib.rgd_rms_bwd_workspace(B, T1, C1, T2, C2)
+    wbuf = torch.empty(max(ws, 1), dtype=torch.uint8, device="cuda")
     if T2 == 0:
         def fwd(i):
             assert lib.rgd_rms_fwd(B, T1, C1, t3(x1[i]), t3(w1, 0), t3(y1[i]), code, code, 1e-6, st) == 0, lib.rgd_last_error()
 
         def bwd(i):
             assert lib.rgd_rms_bwd(B, T1, C1, t3(d1[i]), t3(x1[i]), t3(w1, 0), t3(y1[i]), t3(dw1, 0), 1, code, code, 1e-6,
-                                   wbuf.data_ptr(), ws.value, cbuf.data_ptr(), ct.value, st) == 0, lib.rgd_last_error()
+                                   wbuf.data_ptr(), ws, st) == 0, lib.rgd_last_error()
     else:
         def fwd(i):
             assert lib.rgd_fused_rms_fwd(B, T1, C1, T2, C2, t3(x1[i]), t3(w1, 0), t3(y1[i]), t3(x2[i]), t3(w2, 0), t3(y2[i]),
@@ -453,7 +451,7 @@ def rms_case(torch, name, B, shapes, dtype, nsets, with_api=True, with_cpu=False
         def bwd(i):
             assert lib.rgd_fused_rms_bwd(B, T1, C1, T2, C2, t3(d1[i]), t3(x1[i]), t3(w1, 0), t3(y1[i]), t3(dw1, 0), 1,
                                          t3(d2[i]), t3(x2[i]), t3(w2, 0), t3(y2[i]), t3(dw2, 0), 1, code, code, code, 1e-6,
-                                         wbuf.data_ptr(), ws.value, cbuf.data_ptr(), ct.value, st) == 0, lib.rgd_last_error()
+                                         wbuf.data_ptr(), ws, st) == 0, lib.rgd_last_error()
     n = B * (T1 * C1 + T2 * C2) * es
     api = None
     if with_api:

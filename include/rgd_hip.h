@@ -15,7 +15,11 @@
  *     work and return; they never synchronise.
  *   - return value 0 on success, negative rgd_status otherwise; rgd_last_error() returns a
  *     thread-local message for the last failure on the calling thread.
- *   - functions are re-entrant; the only state is the loaded code object.
+ *   - functions are re-entrant; the only state is the loaded code object and what rgd_init() caches.
+ *   - stream capture: after rgd_init() has returned, every entry point makes no runtime call other than its
+ *     kernel launches on `stream` (no allocation, copy, memset, attribute or device query, no
+ *     hipGetLastError), so a sequence of calls may be recorded into a HIP graph.  The workspace queries
+ *     (rgd_*_workspace, rgd_attn_seqlen_q_rounded) and rgd_version / rgd_last_error touch no stream at all.
  */
 #ifndef RGD_HIP_H
 #define RGD_HIP_H
@@ -58,9 +62,15 @@ typedef struct rgd_tensor4 {
     int64_t stride_n;
 } rgd_tensor4;
 
-/* library / ABI version (major*1000 + minor) and last error text */
+/* library / ABI version (major*1000 + minor) and last error text.  No counterpart in the reference. */
 int         rgd_version(void);
 const char* rgd_last_error(void);
+
+/* One-time set-up: caches the compute-unit count of the current device and sets the LDS size attribute of
+ * every attention kernel.  Thread-safe and idempotent; every entry point calls it on its own, so an explicit
+ * call is only needed before the first entry point runs under stream capture (call it when the library is
+ * loaded).  No counterpart in the reference (Triton configures kernels when it compiles them). */
+int rgd_init(void);
 
 /* ------------------------------------------------------------------------------------------
  * RMSNorm  y = x * rsqrt(mean(x^2) + eps) * w        x (B,T,C), w (B,1,C) or shared
@@ -71,26 +81,23 @@ int rgd_rms_fwd(int64_t B, int64_t T, int64_t C,
                 const rgd_tensor3* x, const rgd_tensor3* w, const rgd_tensor3* y,
                 int x_dtype, int w_dtype, float eps, void* stream);
 
-/* Scratch the backward needs for the deterministic dw reduction.
- * *workspace_bytes: size of `workspace` (any contents on entry): one fp32 partial dw row per block, which
- *                   a second small kernel adds in a fixed order.  Calls that may overlap (different
- *                   streams) need separate workspaces.
- * *counter_bytes:   always 0 in this version; the `counters` argument of the backward calls is kept in
- *                   the interface and ignored (it may be null). */
-int rgd_rms_bwd_workspace(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2,
-                          size_t* workspace_bytes, size_t* counter_bytes);
+/* Bytes of scratch the backward needs for the deterministic dw reduction (any contents on entry): one fp32
+ * partial dw row per block, which a second small kernel adds in a fixed order.  Calls that may overlap
+ * (different streams) need separate workspaces.  T2 = C2 = 0 for the one-tensor backward.  Stands where the
+ * reference allocates its lock and bucket buffers, normalization/rmsnorm_cached.py:455-470. */
+size_t rgd_rms_bwd_workspace(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2);
 
 /* replaces _rms_bwd, normalization/rmsnorm_cached.py:406-569 (kernels :106-264 and :269-313):
  *   dx = (dy*w - xhat*mean(xhat*dy*w)) * rrms,   dw[b or shared] = sum_rows xhat*dy.
  * dw is (B,1,C) addressed with dw->stride_b when w_shared == 0, and a single (C) row holding the
  * sum over the batch when w_shared != 0 (the reference sums a (B,1,C) buffer on the host,
- * rmsnorm_cached.py:623-625).  dw is accumulated in fp32, in a fixed order, and stored in w_dtype. */
+ * rmsnorm_cached.py:623-625).  dw is accumulated in fp32, in a fixed order, and stored in w_dtype.
+ * Rows of any width (the reference loops over channel blocks, rmsnorm_cached.py:198-219). */
 int rgd_rms_bwd(int64_t B, int64_t T, int64_t C,
                 const rgd_tensor3* dy, const rgd_tensor3* x, const rgd_tensor3* w,
                 const rgd_tensor3* dx, const rgd_tensor3* dw, int w_shared,
                 int x_dtype, int w_dtype, float eps,
-                void* workspace, size_t workspace_bytes, void* counters, size_t counter_bytes,
-                void* stream);
+                void* workspace, size_t workspace_bytes, void* stream);
 
 /* replaces _fused_rms_fwd, normalization/fused_rmsnorm_cached.py:389-501 (kernel :6-125):
  * the two tensors are normalised in one launch as one virtual tensor; they share B and the dtype,
@@ -107,8 +114,7 @@ int rgd_fused_rms_bwd(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2,
                       const rgd_tensor3* dy2, const rgd_tensor3* x2, const rgd_tensor3* w2,
                       const rgd_tensor3* dx2, const rgd_tensor3* dw2, int w2_shared,
                       int x_dtype, int w1_dtype, int w2_dtype, float eps,
-                      void* workspace, size_t workspace_bytes, void* counters, size_t counter_bytes,
-                      void* stream);
+                      void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * L2 normalize  y = x / max(||x||, eps)              x (B,T,C)

@@ -16,6 +16,7 @@ LIB_PATH = os.environ.get("RGD_HIP_LIB") or os.path.join(_HERE, "librgd_hip.so")
 HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "rgd_hip.h")
 
 RGD_F32, RGD_F16, RGD_BF16 = 0, 1, 2
+ABI_MAJOR = 2  # rgd_version() // 1000 this binding was written for
 BIAS_NONE, BIAS_VECTOR, BIAS_MATRIX = 0, 1, 2
 
 _DTYPE_CODE = {torch.float32: RGD_F32, torch.float16: RGD_F16, torch.bfloat16: RGD_BF16}
@@ -37,12 +38,13 @@ _T3, _T4 = ctypes.POINTER(Tensor3), ctypes.POINTER(Tensor4)
 _SIGNATURES = {
     "rgd_version": (_int, []),
     "rgd_last_error": (ctypes.c_char_p, []),
+    "rgd_init": (_int, []),
     "rgd_rms_fwd": (_int, [_i64, _i64, _i64, _T3, _T3, _T3, _int, _int, _f32, _vp]),
-    "rgd_rms_bwd_workspace": (_int, [_i64] * 5 + [ctypes.POINTER(_sz), ctypes.POINTER(_sz)]),
-    "rgd_rms_bwd": (_int, [_i64, _i64, _i64, _T3, _T3, _T3, _T3, _T3, _int, _int, _int, _f32, _vp, _sz, _vp, _sz, _vp]),
+    "rgd_rms_bwd_workspace": (_sz, [_i64] * 5),
+    "rgd_rms_bwd": (_int, [_i64, _i64, _i64, _T3, _T3, _T3, _T3, _T3, _int, _int, _int, _f32, _vp, _sz, _vp]),
     "rgd_fused_rms_fwd": (_int, [_i64] * 5 + [_T3] * 6 + [_int, _int, _int, _f32, _vp]),
     "rgd_fused_rms_bwd": (_int, [_i64] * 5 + [_T3] * 5 + [_int] + [_T3] * 5 + [_int] + [_int, _int, _int, _f32,
-                                                                                 _vp, _sz, _vp, _sz, _vp]),
+                                                                                 _vp, _sz, _vp]),
     "rgd_l2_fwd": (_int, [_i64, _i64, _i64, _T3, _T3, _int, _f32, _vp]),
     "rgd_l2_bwd": (_int, [_i64, _i64, _i64, _T3, _T3, _T3, _int, _f32, _vp]),
     "rgd_fused_l2_fwd": (_int, [_i64] * 5 + [_T3] * 4 + [_int, _f32, _vp]),
@@ -89,6 +91,15 @@ def lib():
                 fn = getattr(handle, name)  # AttributeError if the library does not export it
                 fn.restype = res
                 fn.argtypes = args
+            if handle.rgd_version() // 1000 != ABI_MAJOR:
+                raise RuntimeError(f"{LIB_PATH} has ABI version {handle.rgd_version()}, this package needs "
+                                   f"{ABI_MAJOR}xxx: rebuild it")
+            # one-time set-up now (kernel attributes, device properties), so that no entry point has any left to
+            # do when it first runs, e.g. under stream capture.  Without a GPU the call only records that.
+            if torch.cuda.is_available():
+                rc = handle.rgd_init()
+                if rc != 0:
+                    raise RuntimeError(f"rgd_init failed ({rc}): {handle.rgd_last_error().decode(errors='replace')}")
             _lib = handle
     return _lib
 
@@ -120,17 +131,10 @@ def stream_ptr(device):
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
-# scratch buffers (torch-owned), one set per (device, stream): calls on one stream are ordered, so a
-# buffer can be reused by the next call; different streams never share one
-_scratch = {}
-
-
-def scratch(device, kind, nbytes, zero=False):
-    key = (device.index if device.index is not None else torch.cuda.current_device(),
-           torch.cuda.current_stream(device).cuda_stream, kind)
-    buf = _scratch.get(key)
-    if buf is None or buf.numel() < nbytes:
-        n = max(int(nbytes), 256)
-        buf = (torch.zeros if zero else torch.empty)(n, dtype=torch.uint8, device=device)
-        _scratch[key] = buf
-    return buf
+def workspace(device, nbytes):
+    """Scratch for ONE call: a fresh uint8 tensor from PyTorch's caching allocator.  The allocator hands a freed
+    block only to later work of the same stream, so the buffer is safe to drop as soon as the call has been
+    enqueued, calls on different streams or host threads never share one, and under graph capture the block
+    comes from the graph's private pool (the reference allocates delta and dq_accum per call in the same way,
+    flash_attn/flash_attn_triton_cached.py:896-900)."""
+    return torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=device)

@@ -10,7 +10,6 @@
 template <typename T> int dispatch_fwd(const AttnFwdParams& p, unsigned grid, hipStream_t s);
 template <typename T> int dispatch_fwd_merge(const AttnFwdParams& p, unsigned items, hipStream_t s);
 template <typename T> int dispatch_bwd_merge(const AttnBwdParams& p, unsigned items, int nt, hipStream_t s);
-int rgd_num_cus();  // api.hip
 template <typename T, bool DQ> int dispatch_bwd(const AttnBwdParams& p, unsigned grid, hipStream_t s);
 
 namespace {
@@ -46,6 +45,8 @@ constexpr AttnSplitModel kBwdSplit = {1.05f, 1.05f, 1.4f};
 
 int check_common(const char* name, int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, int dtype, int bias_kind,
                  int bias_dtype, const rgd_tensor4* bias) {
+    const int init_rc = rgd_ensure_init();
+    if (init_rc != RGD_OK) return init_rc;
     RGD_REQUIRE(dtype == RGD_F16 || dtype == RGD_BF16, RGD_ERR_INVALID, "%s: Only support fp16 and bf16", name);
     RGD_REQUIRE(D >= 1 && D <= 128, RGD_ERR_INVALID, "%s: FlashAttention only support head dimensions up to 128", name);
     RGD_REQUIRE(B >= 0 && H >= 0 && Tq >= 0 && Tk >= 0, RGD_ERR_INVALID, "%s: negative shape", name);
@@ -136,13 +137,11 @@ int rgd_attn_fwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
     hipStream_t s = static_cast<hipStream_t>(stream);
     rc = dtype == RGD_F16 ? dispatch_fwd<f16_t>(p, (unsigned)grid, s) : dispatch_fwd<bf16_t>(p, (unsigned)grid, s);
     if (rc != RGD_OK) return rc;
-    RGD_CHECK_LAUNCH(name);
     if (plan.s > 1) {
         const unsigned n = (unsigned)plan.items_split(items);
         rc = dtype == RGD_F16 ? dispatch_fwd_merge<f16_t>(p, n, s) : dispatch_fwd_merge<bf16_t>(p, n, s);
         if (rc != RGD_OK) return rc;
-        RGD_CHECK_LAUNCH(name);
-    }
+        }
     return RGD_OK;
 }
 
@@ -165,6 +164,10 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
     for (const rgd_tensor4* t : all) RGD_REQUIRE(t, RGD_ERR_INVALID, "%s: null tensor descriptor", name);
     RGD_REQUIRE(Tq == 0 || (dout->ptr && q->ptr && o->ptr && dq->ptr && lse), RGD_ERR_INVALID, "%s: null tensor", name);
     RGD_REQUIRE(Tk == 0 || (k->ptr && v->ptr && dk->ptr && dv->ptr), RGD_ERR_INVALID, "%s: null tensor", name);
+    // offsets inside one staged tile (K, V in the dQ kernel; Q, dO in the dK/dV kernel) are kept in 32 bits
+    for (const rgd_tensor4* t : {q, k, v, dout})
+        RGD_REQUIRE(llabs(t->stride_n) < (1ll << 24), RGD_ERR_UNSUPPORTED, "%s: token stride %lld is outside (-2^24, 2^24)",
+                    name, (long long)t->stride_n);
     // delta is required; whatever the workspace holds beyond it is used to split the last round of workgroups
     const size_t delta_bytes = bwd_delta_bytes(B, H, Tq);
     RGD_REQUIRE(workspace_bytes >= delta_bytes && (workspace || Tq == 0), RGD_ERR_WORKSPACE, "%s: workspace too small",
@@ -222,13 +225,11 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
         RGD_REQUIRE(grid < (1ll << 31), RGD_ERR_UNSUPPORTED, "%s: grid too large", name);
         rc = dtype == RGD_F16 ? dispatch_bwd<f16_t, true>(p, (unsigned)grid, s) : dispatch_bwd<bf16_t, true>(p, (unsigned)grid, s);
         if (rc != RGD_OK) return rc;
-        RGD_CHECK_LAUNCH(name);
-        if (plan.s > 1) {
+            if (plan.s > 1) {
             const unsigned n = (unsigned)plan.items_split(items);
             rc = dtype == RGD_F16 ? dispatch_bwd_merge<f16_t>(p, n, 1, s) : dispatch_bwd_merge<bf16_t>(p, n, 1, s);
             if (rc != RGD_OK) return rc;
-            RGD_CHECK_LAUNCH(name);
-        }
+                }
     }
     if (Tk > 0) {  // dK and dV (reads delta)
         p.nblk = (int)((Tk + BWD_BM - 1) / BWD_BM);
@@ -244,13 +245,11 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
         RGD_REQUIRE(grid < (1ll << 31), RGD_ERR_UNSUPPORTED, "%s: grid too large", name);
         rc = dtype == RGD_F16 ? dispatch_bwd<f16_t, false>(p, (unsigned)grid, s) : dispatch_bwd<bf16_t, false>(p, (unsigned)grid, s);
         if (rc != RGD_OK) return rc;
-        RGD_CHECK_LAUNCH(name);
-        if (plan.s > 1) {
+            if (plan.s > 1) {
             const unsigned n = (unsigned)plan.items_split(items);
             rc = dtype == RGD_F16 ? dispatch_bwd_merge<f16_t>(p, n, 2, s) : dispatch_bwd_merge<bf16_t>(p, n, 2, s);
             if (rc != RGD_OK) return rc;
-            RGD_CHECK_LAUNCH(name);
-        }
+                }
     }
     return RGD_OK;
 }

@@ -5,3 +5,4 @@ template int dispatch_fwd_merge<bf16_t>(const AttnFwdParams&, unsigned, hipStrea
 template int dispatch_bwd<bf16_t, true>(const AttnBwdParams&, unsigned, hipStream_t);
 template int dispatch_bwd<bf16_t, false>(const AttnBwdParams&, unsigned, hipStream_t);
 template int dispatch_bwd_merge<bf16_t>(const AttnBwdParams&, unsigned, int, hipStream_t);
+template int attn_configure_all<bf16_t>();

@@ -5,3 +5,4 @@ template int dispatch_fwd_merge<f16_t>(const AttnFwdParams&, unsigned, hipStream
 template int dispatch_bwd<f16_t, true>(const AttnBwdParams&, unsigned, hipStream_t);
 template int dispatch_bwd<f16_t, false>(const AttnBwdParams&, unsigned, hipStream_t);
 template int dispatch_bwd_merge<f16_t>(const AttnBwdParams&, unsigned, int, hipStream_t);
+template int attn_configure_all<f16_t>();

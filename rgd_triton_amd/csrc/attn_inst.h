@@ -6,25 +6,13 @@
 #include "attn_bwd.h"
 
 template <typename T, int DPAD, int BIAS> int launch_fwd(const AttnFwdParams& p, unsigned grid, hipStream_t s) {
-    auto kern = attn_fwd_kernel<T, DPAD, BIAS>;
-    constexpr size_t lds = AttnFwdSmem<DPAD>::BYTES;
-    static bool configured = false;  // benign race: the attribute is idempotent
-    if (!configured && lds > 48 * 1024) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)lds) != hipSuccess) {
-            rgd_set_error("rgd_attn_fwd: cannot reserve %zu bytes of LDS", lds);
-            return RGD_ERR_LAUNCH;
-        }
-        configured = true;
-    }
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(ATTN_THREADS), lds, s, p);
-    return RGD_OK;
+    constexpr size_t lds = AttnFwdSmem<DPAD>::BYTES;  // its attribute was set by attn_configure_all
+    return rgd_launch_status("rgd_attn_fwd", rgd_launch(attn_fwd_kernel<T, DPAD, BIAS>, dim3(grid), dim3(ATTN_THREADS), lds, s, p));
 }
 
 template <typename T, int DPAD> int launch_fwd_merge(const AttnFwdParams& p, unsigned items, hipStream_t s) {
     const unsigned gy = (ATTN_BM * (DPAD / 4) + 255) / 256;
-    hipLaunchKernelGGL((attn_fwd_merge_kernel<T, DPAD>), dim3(items, gy), dim3(256), 0, s, p);
-    return RGD_OK;
+    return rgd_launch_status("rgd_attn_fwd (merge)", rgd_launch(attn_fwd_merge_kernel<T, DPAD>, dim3(items, gy), dim3(256), 0, s, p));
 }
 
 template <typename T> int dispatch_fwd_merge(const AttnFwdParams& p, unsigned items, hipStream_t s) {
@@ -52,17 +40,7 @@ template <typename T> int dispatch_fwd(const AttnFwdParams& p, unsigned grid, hi
 template <typename T, int DPAD, int BIAS, bool DQ> int launch_bwd(const AttnBwdParams& p, unsigned grid, hipStream_t s) {
     auto kern = DQ ? attn_bwd_dq_kernel<T, DPAD, BIAS> : attn_bwd_dkv_kernel<T, DPAD, BIAS>;
     constexpr size_t lds = DQ ? DqSmem<DPAD>::BYTES : DkvSmem<DPAD, dkv_nsub(DPAD, BIAS)>::BYTES;
-    static bool configured = false;
-    if (!configured && lds > 48 * 1024) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)lds) != hipSuccess) {
-            rgd_set_error("rgd_attn_bwd: cannot reserve %zu bytes of LDS", lds);
-            return RGD_ERR_LAUNCH;
-        }
-        configured = true;
-    }
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(BWD_THREADS), lds, s, p);
-    return RGD_OK;
+    return rgd_launch_status("rgd_attn_bwd", rgd_launch(kern, dim3(grid), dim3(BWD_THREADS), lds, s, p));
 }
 
 template <typename T, bool DQ> int dispatch_bwd(const AttnBwdParams& p, unsigned grid, hipStream_t s) {
@@ -83,8 +61,7 @@ template <typename T, bool DQ> int dispatch_bwd(const AttnBwdParams& p, unsigned
 
 template <typename T, int DPAD> int launch_bwd_merge(const AttnBwdParams& p, unsigned items, int nt, hipStream_t s) {
     const unsigned gy = (BWD_BM * (DPAD / 4) + 255) / 256;
-    hipLaunchKernelGGL((attn_bwd_merge_kernel<T, DPAD>), dim3(items, gy, nt), dim3(256), 0, s, p, nt);
-    return RGD_OK;
+    return rgd_launch_status("rgd_attn_bwd (merge)", rgd_launch(attn_bwd_merge_kernel<T, DPAD>, dim3(items, gy, nt), dim3(256), 0, s, p, nt));
 }
 
 template <typename T> int dispatch_bwd_merge(const AttnBwdParams& p, unsigned items, int nt, hipStream_t s) {
@@ -92,4 +69,42 @@ template <typename T> int dispatch_bwd_merge(const AttnBwdParams& p, unsigned it
     if (p.D <= 64) return launch_bwd_merge<T, 64>(p, items, nt, s);
     if (p.D <= 96) return launch_bwd_merge<T, 96>(p, items, nt, s);
     return launch_bwd_merge<T, 128>(p, items, nt, s);
+}
+
+// Kernels that use more than 48 KB of dynamic LDS need hipFuncAttributeMaxDynamicSharedMemorySize before their first
+// launch.  Called once per process from the library's set-up, for every instantiation of this element type, so no
+// entry point touches function attributes afterwards (an entry point may run under stream capture, where such a
+// call is not allowed).
+template <typename T, int DPAD, int BIAS> int attn_configure_one() {
+    struct K {
+        const void* fn;
+        size_t lds;
+    };
+    const K ks[] = {
+        {reinterpret_cast<const void*>(attn_fwd_kernel<T, DPAD, BIAS>), AttnFwdSmem<DPAD>::BYTES},
+        {reinterpret_cast<const void*>(attn_bwd_dq_kernel<T, DPAD, BIAS>), DqSmem<DPAD>::BYTES},
+        {reinterpret_cast<const void*>(attn_bwd_dkv_kernel<T, DPAD, BIAS>), DkvSmem<DPAD, dkv_nsub(DPAD, BIAS)>::BYTES},
+    };
+    for (const K& k : ks) {
+        if (k.lds <= 48 * 1024) continue;
+        if (hipFuncSetAttribute(k.fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)k.lds) != hipSuccess) {
+            (void)hipGetLastError();
+            rgd_set_error("rgd_init: cannot reserve %zu bytes of LDS for an attention kernel", k.lds);
+            return RGD_ERR_LAUNCH;
+        }
+    }
+    return RGD_OK;
+}
+template <typename T, int DPAD> int attn_configure_dpad() {
+    int rc = attn_configure_one<T, DPAD, BIAS_OFF>();
+    if (rc == RGD_OK) rc = attn_configure_one<T, DPAD, BIAS_SAME>();
+    if (rc == RGD_OK) rc = attn_configure_one<T, DPAD, BIAS_F32>();
+    return rc;
+}
+template <typename T> int attn_configure_all() {
+    int rc = attn_configure_dpad<T, 32>();
+    if (rc == RGD_OK) rc = attn_configure_dpad<T, 64>();
+    if (rc == RGD_OK) rc = attn_configure_dpad<T, 96>();
+    if (rc == RGD_OK) rc = attn_configure_dpad<T, 128>();
+    return rc;
 }

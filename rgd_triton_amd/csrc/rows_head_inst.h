@@ -9,10 +9,8 @@ static int head_launch_one(const HeadParams& p, dim3 grid, hipStream_t s) {
     constexpr int U = head_unroll(MODE, NV);
     // rows that fill their lane group exactly (the power-of-two head dims) skip every range mask
     if (VECTOR && p.D == G * NV * VEC)
-        hipLaunchKernelGGL((head_rows_kernel<T, TP, MODE, G, NV, VEC, VECTOR, VECTOR, U>), grid, dim3(256), 0, s, p);
-    else
-        hipLaunchKernelGGL((head_rows_kernel<T, TP, MODE, G, NV, VEC, VECTOR, false, U>), grid, dim3(256), 0, s, p);
-    return 0;
+        return rgd_launch_status("head rows", rgd_launch(head_rows_kernel<T, TP, MODE, G, NV, VEC, VECTOR, VECTOR, U>, grid, dim3(256), 0, s, p));
+    return rgd_launch_status("head rows", rgd_launch(head_rows_kernel<T, TP, MODE, G, NV, VEC, VECTOR, false, U>, grid, dim3(256), 0, s, p));
 }
 
 template <typename T, typename TP, int MODE, bool VECTOR>

@@ -234,7 +234,11 @@ __global__ __launch_bounds__(NW * 64) void wide_rows_kernel(const WideParams p) 
 // row statistics, the second re-reads x (and dy, w) -- the row was just read, so this comes from L2 -- and
 // writes the result.  Only the dw sums of the RMSNorm backward stay in registers (NKW chunks per lane, a
 // compile-time bound; 0 when there is no dw); since every channel belongs to exactly one lane of the
-// workgroup, the block's partial dw row is written straight from them.
+// workgroup, the block's partial dw row is written straight from them.  Rows with more than NKW chunks per
+// lane are covered by gridDim.z channel slabs of 256 * NKW * VEC channels: the blocks of slab 0 do everything
+// above and keep the dw sums of the first slab, the blocks of slab z > 0 recompute the row statistic from x and
+// keep the dw sums of their own slab only (they write no dx), so any width works and every sum keeps its
+// fixed order.
 template <typename T, int OP, bool BWD, int VEC, bool VECTOR, int NKW>
 __global__ __launch_bounds__(256) void wide_stream_kernel(const WideParams p) {
     __shared__ float s_red[2][2][4];  // [parity][statistic][wavefront]
@@ -248,6 +252,9 @@ __global__ __launch_bounds__(256) void wide_stream_kernel(const WideParams p) {
     const int r1 = min(h.T, r0 + p.rows_per_chunk);
     const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6;
     const int nk = (C + 256 * VEC - 1) / (256 * VEC);  // chunks per lane
+    const int k0 = NKW > 0 ? (int)blockIdx.z * NKW : 0;  // first chunk of this block's dw slab
+    const bool lead = blockIdx.z == 0;                    // this block also produces dx
+    if (k0 >= nk) return;  // the narrower of two tensors may have fewer slabs (block-uniform)
 
     const T* xb = static_cast<const T*>(h.x) + (int64_t)b * h.sx_b;
     const T* db = BWD ? static_cast<const T*>(h.dy) + (int64_t)b * h.sd_b : nullptr;
@@ -278,13 +285,17 @@ __global__ __launch_bounds__(256) void wide_stream_kernel(const WideParams p) {
             float xv[VEC], dv[VEC], wv[VEC];
             load_chunk<T, VEC, VECTOR>(xr, first, C, xv);
             if constexpr (BWD) {
-                load_chunk<T, VEC, VECTOR>(dr, first, C, dv);
-                if constexpr (HAS_W) load_w(first, wv);
+                if (lead) {
+                    load_chunk<T, VEC, VECTOR>(dr, first, C, dv);
+                    if constexpr (HAS_W) load_w(first, wv);
+                }
             }
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
                 ss += xv[e] * xv[e];
-                if constexpr (BWD) sd += xv[e] * (HAS_W ? dv[e] * wv[e] : dv[e]);
+                if constexpr (BWD) {
+                    if (lead) sd += xv[e] * (HAS_W ? dv[e] * wv[e] : dv[e]);
+                }
             }
         }
         ss = group_reduce<64>(ss);
@@ -327,9 +338,26 @@ __global__ __launch_bounds__(256) void wide_stream_kernel(const WideParams p) {
             store_chunk<T, VEC, VECTOR>(yr, first, C, out);
         };
         if constexpr (NKW > 0) {
+            if (lead) {
 #pragma unroll
-            for (int k = 0; k < NKW; ++k)
-                if (k < nk) body(k, dwacc[k]);
+                for (int k = 0; k < NKW; ++k)
+                    if (k < nk) body(k, dwacc[k]);
+                float unused[VEC] = {};
+                for (int k = NKW; k < nk; ++k) body(k, unused);  // chunks whose dw sums belong to later slabs
+            } else {
+                // dw sums of this slab only: xhat * dy
+#pragma unroll
+                for (int k = 0; k < NKW; ++k) {
+                    if (k0 + k < nk) {
+                        const int first = ((k0 + k) * 256 + tid) * VEC;
+                        float xv[VEC], dv[VEC];
+                        load_chunk<T, VEC, VECTOR>(xr, first, C, xv);
+                        load_chunk<T, VEC, VECTOR>(dr, first, C, dv);
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) dwacc[k][e] += xv[e] * rn * dv[e];
+                    }
+                }
+            }
         } else {
             for (int k = 0; k < nk; ++k) body(k, dwacc[0]);
         }
@@ -344,7 +372,7 @@ __global__ __launch_bounds__(256) void wide_stream_kernel(const WideParams p) {
         for (int k = 0; k < NKW; ++k)
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
-                const int c = (k * 256 + tid) * VEC + e;
+                const int c = ((k0 + k) * 256 + tid) * VEC + e;
                 if (c < C) {
                     if (h.nleaf == 1)
                         store_dyn(dw_row, h.w_dtype, c, dwacc[k][e]);
@@ -368,9 +396,8 @@ struct WideHalfArgs {
 };
 
 int wide_launch(const char* name, int op, bool bwd, int64_t B, const WideHalfArgs& a1, const WideHalfArgs& a2,
-                int dtype, float eps, void* workspace, size_t workspace_bytes, void* counters,
-                size_t counter_bytes, void* stream);
-int wide_workspace(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2, size_t* ws, size_t* ctr);
+                int dtype, float eps, void* workspace, size_t workspace_bytes, void* stream);
+size_t wide_workspace(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2);
 
 // per-dtype instantiation units (rows_wide_f32.hip, rows_wide_f16.hip, rows_wide_bf16.hip)
 struct WideConfig {

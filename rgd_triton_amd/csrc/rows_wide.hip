@@ -5,8 +5,6 @@
 #include <algorithm>
 #include <string.h>
 
-int rgd_num_cus();  // api.hip
-
 #ifndef RGD_DW_BLOCKS_PER_CU
 #define RGD_DW_BLOCKS_PER_CU 1
 #endif
@@ -71,19 +69,16 @@ bool t3_vec_ok(const rgd_tensor3* t, int es) {
 
 }  // namespace
 
-int wide_workspace(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2, size_t* ws, size_t* ctr) {
+size_t wide_workspace(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2) {
     const int64_t target = (int64_t)rgd_num_cus() * DW_BLOCKS_PER_CU;
     const size_t r1 = half_bound(B, T1, target), r2 = half_bound(B, T2, target);
-    *ws = (r1 * (size_t)std::max<int64_t>(C1, 0) + r2 * (size_t)std::max<int64_t>(C2, 0)) * sizeof(float);
-    *ctr = 0;  // no counters are needed; the argument stays in the interface
-    return RGD_OK;
+    return (r1 * (size_t)std::max<int64_t>(C1, 0) + r2 * (size_t)std::max<int64_t>(C2, 0)) * sizeof(float);
 }
 
 int wide_launch(const char* name, int op, bool bwd, int64_t B, const WideHalfArgs& a1, const WideHalfArgs& a2,
-                int dtype, float eps, void* workspace, size_t workspace_bytes, void* counters,
-                size_t counter_bytes, void* stream) {
-    (void)counters;  // kept in the interface, not used
-    (void)counter_bytes;
+                int dtype, float eps, void* workspace, size_t workspace_bytes, void* stream) {
+    const int init_rc = rgd_ensure_init();
+    if (init_rc != RGD_OK) return init_rc;
     RGD_REQUIRE(rgd_dtype_ok(dtype), RGD_ERR_INVALID, "%s: Only support fp16, bf16, and fp32", name);
     RGD_REQUIRE(B >= 0 && B <= 65535, RGD_ERR_INVALID, "%s: batch %lld out of range", name, (long long)B);
     const WideHalfArgs* as[2] = {&a1, &a2};
@@ -141,11 +136,13 @@ int wide_launch(const char* name, int op, bool bwd, int64_t B, const WideHalfArg
         }
     }
     cfg.stream = cfg.NV == 0;  // too wide for registers: the two-pass streaming kernel
+    int64_t slabs = 1;  // channel slabs of the streaming RMSNorm backward (its dw sums stay in registers, slab by slab)
     if (cfg.stream) {
-        const int64_t dw_limit = (int64_t)256 * wide_stream_nkw(vec) * vec;  // dw sums stay in registers
-        RGD_REQUIRE(!(has_w && bwd) || maxC <= dw_limit, RGD_ERR_UNSUPPORTED,
-                    "%s: rows of %lld elements exceed the limit of the backward (%lld)", name, (long long)maxC,
-                    (long long)dw_limit);
+        if (has_w && bwd) {
+            const int64_t slab_channels = (int64_t)256 * wide_stream_nkw(vec) * vec;
+            slabs = (maxC + slab_channels - 1) / slab_channels;
+            RGD_REQUIRE(slabs <= 65535, RGD_ERR_UNSUPPORTED, "%s: rows of %lld elements are too wide", name, (long long)maxC);
+        }
         cfg.G = 64;
         cfg.NV = 1;
         cfg.WPR = 4;
@@ -217,7 +214,7 @@ int wide_launch(const char* name, int op, bool bwd, int64_t B, const WideHalfArg
     }
     RGD_REQUIRE(grid_x < (1ll << 31), RGD_ERR_UNSUPPORTED, "%s: grid too large", name);
 
-    const dim3 grid((unsigned)grid_x, (unsigned)B, 1);
+    const dim3 grid((unsigned)grid_x, (unsigned)B, (unsigned)slabs);
     // one row of dw sums per wavefront group (the streaming kernel writes its sums from registers)
     const size_t lds = (tree && !cfg.stream) ? (size_t)(NW / cfg.WPR) * maxC * sizeof(float) : 0;
     RGD_REQUIRE(lds <= 64 * 1024, RGD_ERR_UNSUPPORTED, "%s: row too wide for the dw staging buffer", name);
@@ -230,11 +227,8 @@ int wide_launch(const char* name, int op, bool bwd, int64_t B, const WideHalfArg
     else
         rc = wide_dispatch<bf16_t>(cfg, p, grid, lds, s);
     if (rc != RGD_OK) return rc;
-    RGD_CHECK_LAUNCH(name);
-    if (red_grid > 0) {  // dw = fixed-order sum of the blocks' partial rows
-        hipLaunchKernelGGL(wide_dw_reduce_kernel, dim3((unsigned)red_grid), dim3(WIDE_RED_WAVES * 64), 0, s, p);
-        RGD_CHECK_LAUNCH(name);
-    }
+    if (red_grid > 0)  // dw = fixed-order sum of the blocks' partial rows
+        return rgd_launch_status(name, rgd_launch(wide_dw_reduce_kernel, dim3((unsigned)red_grid), dim3(WIDE_RED_WAVES * 64), 0, s, p));
     return RGD_OK;
 }
 
@@ -265,65 +259,59 @@ extern "C" {
 int rgd_rms_fwd(int64_t B, int64_t T, int64_t C, const rgd_tensor3* x, const rgd_tensor3* w, const rgd_tensor3* y,
                 int x_dtype, int w_dtype, float eps, void* stream) {
     return wide_launch("rgd_rms_fwd", WIDE_RMS, false, B, half(T, C, x, nullptr, y, w, nullptr, w_dtype), kNoHalf,
-                       x_dtype, eps, nullptr, 0, nullptr, 0, stream);
+                       x_dtype, eps, nullptr, 0, stream);
 }
 
-int rgd_rms_bwd_workspace(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2, size_t* workspace_bytes,
-                          size_t* counter_bytes) {
-    RGD_REQUIRE(workspace_bytes && counter_bytes, RGD_ERR_INVALID, "rgd_rms_bwd_workspace: null output");
-    return wide_workspace(B, T1, C1, T2, C2, workspace_bytes, counter_bytes);
+size_t rgd_rms_bwd_workspace(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2) {
+    return wide_workspace(B, T1, C1, T2, C2);
 }
 
 int rgd_rms_bwd(int64_t B, int64_t T, int64_t C, const rgd_tensor3* dy, const rgd_tensor3* x, const rgd_tensor3* w,
                 const rgd_tensor3* dx, const rgd_tensor3* dw, int w_shared, int x_dtype, int w_dtype, float eps,
-                void* workspace, size_t workspace_bytes, void* counters, size_t counter_bytes, void* stream) {
+                void* workspace, size_t workspace_bytes, void* stream) {
     return wide_launch("rgd_rms_bwd", WIDE_RMS, true, B, half(T, C, x, dy, dx, w, dw, w_dtype, w_shared), kNoHalf,
-                       x_dtype, eps, workspace, workspace_bytes, counters, counter_bytes, stream);
+                       x_dtype, eps, workspace, workspace_bytes, stream);
 }
 
 int rgd_fused_rms_fwd(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2, const rgd_tensor3* x1,
                       const rgd_tensor3* w1, const rgd_tensor3* y1, const rgd_tensor3* x2, const rgd_tensor3* w2,
                       const rgd_tensor3* y2, int x_dtype, int w1_dtype, int w2_dtype, float eps, void* stream) {
     return wide_launch("rgd_fused_rms_fwd", WIDE_RMS, false, B, half(T1, C1, x1, nullptr, y1, w1, nullptr, w1_dtype),
-                       half(T2, C2, x2, nullptr, y2, w2, nullptr, w2_dtype), x_dtype, eps, nullptr, 0, nullptr, 0,
-                       stream);
+                       half(T2, C2, x2, nullptr, y2, w2, nullptr, w2_dtype), x_dtype, eps, nullptr, 0, stream);
 }
 
 int rgd_fused_rms_bwd(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2, const rgd_tensor3* dy1,
                       const rgd_tensor3* x1, const rgd_tensor3* w1, const rgd_tensor3* dx1, const rgd_tensor3* dw1,
                       int w1_shared, const rgd_tensor3* dy2, const rgd_tensor3* x2, const rgd_tensor3* w2,
                       const rgd_tensor3* dx2, const rgd_tensor3* dw2, int w2_shared, int x_dtype, int w1_dtype,
-                      int w2_dtype, float eps, void* workspace, size_t workspace_bytes, void* counters,
-                      size_t counter_bytes, void* stream) {
+                      int w2_dtype, float eps, void* workspace, size_t workspace_bytes, void* stream) {
     return wide_launch("rgd_fused_rms_bwd", WIDE_RMS, true, B, half(T1, C1, x1, dy1, dx1, w1, dw1, w1_dtype, w1_shared),
                        half(T2, C2, x2, dy2, dx2, w2, dw2, w2_dtype, w2_shared), x_dtype, eps, workspace,
-                       workspace_bytes, counters, counter_bytes, stream);
+                       workspace_bytes, stream);
 }
 
 int rgd_l2_fwd(int64_t B, int64_t T, int64_t C, const rgd_tensor3* x, const rgd_tensor3* y, int dtype, float eps,
                void* stream) {
-    return wide_launch("rgd_l2_fwd", WIDE_L2, false, B, half(T, C, x, nullptr, y), kNoHalf, dtype, eps, nullptr, 0,
-                       nullptr, 0, stream);
+    return wide_launch("rgd_l2_fwd", WIDE_L2, false, B, half(T, C, x, nullptr, y), kNoHalf, dtype, eps, nullptr, 0, stream);
 }
 
 int rgd_l2_bwd(int64_t B, int64_t T, int64_t C, const rgd_tensor3* dy, const rgd_tensor3* x, const rgd_tensor3* dx,
                int dtype, float eps, void* stream) {
-    return wide_launch("rgd_l2_bwd", WIDE_L2, true, B, half(T, C, x, dy, dx), kNoHalf, dtype, eps, nullptr, 0, nullptr,
-                       0, stream);
+    return wide_launch("rgd_l2_bwd", WIDE_L2, true, B, half(T, C, x, dy, dx), kNoHalf, dtype, eps, nullptr, 0, stream);
 }
 
 int rgd_fused_l2_fwd(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2, const rgd_tensor3* x1,
                      const rgd_tensor3* y1, const rgd_tensor3* x2, const rgd_tensor3* y2, int dtype, float eps,
                      void* stream) {
     return wide_launch("rgd_fused_l2_fwd", WIDE_L2, false, B, half(T1, C1, x1, nullptr, y1),
-                       half(T2, C2, x2, nullptr, y2), dtype, eps, nullptr, 0, nullptr, 0, stream);
+                       half(T2, C2, x2, nullptr, y2), dtype, eps, nullptr, 0, stream);
 }
 
 int rgd_fused_l2_bwd(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2, const rgd_tensor3* dy1,
                      const rgd_tensor3* x1, const rgd_tensor3* dx1, const rgd_tensor3* dy2, const rgd_tensor3* x2,
                      const rgd_tensor3* dx2, int dtype, float eps, void* stream) {
     return wide_launch("rgd_fused_l2_bwd", WIDE_L2, true, B, half(T1, C1, x1, dy1, dx1), half(T2, C2, x2, dy2, dx2),
-                       dtype, eps, nullptr, 0, nullptr, 0, stream);
+                       dtype, eps, nullptr, 0, stream);
 }
 
 }  // extern "C"

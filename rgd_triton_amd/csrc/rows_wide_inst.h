@@ -12,9 +12,8 @@ static int wide_launch_one(const WideParams& p, dim3 grid, size_t lds, hipStream
     constexpr int NW = wide_waves(OP, BWD);
     // the host never selects more elements per lane than this (they would not stay in registers)
     if constexpr (NV * VEC <= ((OP == WIDE_RMS && (BWD || !RGD_WIDE_RMS_FWD_64)) ? 32 : 64)) {
-        hipLaunchKernelGGL((wide_rows_kernel<T, OP, BWD, G, NV, VEC, VECTOR, U, NW, WPR>), grid, dim3(NW * 64), lds, s,
-                           p);
-        return 0;
+        return rgd_launch_status("wide rows", rgd_launch(wide_rows_kernel<T, OP, BWD, G, NV, VEC, VECTOR, U, NW, WPR>, grid,
+                                                         dim3(NW * 64), lds, s, p));
     }
     rgd_set_error("wide rows: %d elements per lane were not compiled", NV * VEC);
     return RGD_ERR_UNSUPPORTED;
@@ -56,8 +55,7 @@ template <typename T, int OP, bool BWD, bool VECTOR>
 static int wide_launch_stream(const WideParams& p, dim3 grid, hipStream_t s) {
     constexpr int VEC = VECTOR ? 16 / (int)sizeof(T) : 2;
     constexpr int NKW = (OP == WIDE_RMS && BWD) ? wide_stream_nkw(VEC) : 0;
-    hipLaunchKernelGGL((wide_stream_kernel<T, OP, BWD, VEC, VECTOR, NKW>), grid, dim3(256), 0, s, p);
-    return 0;
+    return rgd_launch_status("wide rows (streaming)", rgd_launch(wide_stream_kernel<T, OP, BWD, VEC, VECTOR, NKW>, grid, dim3(256), 0, s, p));
 }
 
 template <typename T>

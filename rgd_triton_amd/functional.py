@@ -80,14 +80,10 @@ def _check_rows(x):
 
 
 def _rms_scratch(x1, x2):
-    lib = _hip.lib()
-    ws, ct = ctypes.c_size_t(), ctypes.c_size_t()
     B = x1.shape[0]
     T2, C2 = (x2.shape[1], x2.shape[2]) if x2 is not None else (0, 0)
-    _hip.check(lib.rgd_rms_bwd_workspace(B, x1.shape[1], x1.shape[2], T2, C2, ctypes.byref(ws), ctypes.byref(ct)),
-               "rgd_rms_bwd_workspace")
-    # counter_bytes is 0 in this version of the library: the backward takes a null counter buffer
-    return _hip.scratch(x1.device, "rms_ws", ws.value), ws.value
+    nbytes = _hip.lib().rgd_rms_bwd_workspace(B, x1.shape[1], x1.shape[2], T2, C2)
+    return _hip.workspace(x1.device, nbytes), nbytes
 
 
 class RMS_Func(torch.autograd.Function):
@@ -126,7 +122,7 @@ class RMS_Func(torch.autograd.Function):
         lib = _hip.lib()
         _hip.check(lib.rgd_rms_bwd(B, T, C, t3(dy), t3(x), t3(w, w_sb), t3(dx), t3(dw, 0 if shared else dw.stride(0)),
                                    int(shared), _hip.dtype_code(x.dtype), _hip.dtype_code(w.dtype), ctx.norm_eps,
-                                   wbuf.data_ptr(), wsz, None, 0, _hip.stream_ptr(x.device)), "rgd_rms_bwd")
+                                   wbuf.data_ptr(), wsz, _hip.stream_ptr(x.device)), "rgd_rms_bwd")
         return dx, dw, None, None
 
 
@@ -181,7 +177,7 @@ class Fused_RMS_Func(torch.autograd.Function):
             t3(dy1), t3(x1), t3(w1, sb1), t3(dx1), t3(dw1, 0 if s1 else dw1.stride(0)), int(s1),
             t3(dy2), t3(x2), t3(w2, sb2), t3(dx2), t3(dw2, 0 if s2 else dw2.stride(0)), int(s2),
             _hip.dtype_code(x1.dtype), _hip.dtype_code(w1.dtype), _hip.dtype_code(w2.dtype), ctx.norm_eps,
-            wbuf.data_ptr(), wsz, None, 0, _hip.stream_ptr(x1.device)), "rgd_fused_rms_bwd")
+            wbuf.data_ptr(), wsz, _hip.stream_ptr(x1.device)), "rgd_fused_rms_bwd")
         return dx1, dx2, dw1, dw2, None, None
 
 
@@ -492,7 +488,7 @@ def _flash_attn_forward(q, k, v, bias=None, causal=False, softmax_scale=None, ke
     seqlen_q_rounded = lib.rgd_attn_seqlen_q_rounded(seqlen_q)
     lse = torch.empty((batch, nheads, seqlen_q_rounded), device=q.device, dtype=torch.float32)
     o = torch.empty_like(q)
-    ws = _hip.scratch(q.device, "attn_fwd_ws", lib.rgd_attn_fwd_workspace(batch, nheads, seqlen_q, seqlen_k, d))
+    ws = _hip.workspace(q.device, lib.rgd_attn_fwd_workspace(batch, nheads, seqlen_q, seqlen_k, d))
     _hip.check(lib.rgd_attn_fwd(batch, nheads, seqlen_q, seqlen_k, d, t4(q, False), t4(k, False), t4(v, False),
                                 bdesc, bkind, bdtype, t4(o, False), ctypes.c_void_p(lse.data_ptr()),
                                 _hip.dtype_code(q.dtype), int(bool(causal)), float(softmax_scale),
@@ -517,7 +513,7 @@ def _flash_attn_backward(do, q, k, v, o, lse, dq, dk, dv, bias=None, causal=Fals
     softmax_scale = softmax_scale or 1.0 / math.sqrt(d)
     bdesc, bkind, bdtype = _bias_args(bias, q, seqlen_q, seqlen_k, batch, nheads)
     nbytes = lib.rgd_attn_bwd_workspace(batch, nheads, seqlen_q, seqlen_k, d)
-    ws = _hip.scratch(q.device, "attn_ws", nbytes)
+    ws = _hip.workspace(q.device, nbytes)
     _hip.check(lib.rgd_attn_bwd(batch, nheads, seqlen_q, seqlen_k, d, t4(do, False), t4(q, False), t4(k, False),
                                 t4(v, False), t4(o, False), ctypes.c_void_p(lse.data_ptr()), bdesc, bkind, bdtype,
                                 t4(dq, False), t4(dk, False), t4(dv, False), _hip.dtype_code(q.dtype),

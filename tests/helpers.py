@@ -57,3 +57,23 @@ def assert_close_allow_inf(actual, expected, dtype, name=""):
     fin = ~torch.isinf(e)
     rtol, atol = oracle.get_tolerance(dtype)
     torch.testing.assert_close(a[fin], e[fin], rtol=rtol, atol=atol, msg=lambda m: f"{name}: {m}")
+
+
+RACE_ITERS = 250  # repeats of the reference's race-condition tests (tests/test_flash_attn.py:367, tests/test_rms.py:228)
+
+
+def assert_repeats_bit_exact(fn, names, iters=RACE_ITERS):
+    """Runs fn() (which returns GPU tensors) once, then `iters` more times, and requires every tensor of every repeat
+    to have the bits of the first run.  Mismatches are counted on the GPU (integer views, so NaN equals NaN) and
+    read back once at the end: the loop stays as dense as the reference's, which checks on the host every time."""
+    ints = {1: torch.int8, 2: torch.int16, 4: torch.int32, 8: torch.int64}
+    first = [t.detach().clone() for t in fn()]
+    views = [t.view(ints[t.element_size()]) for t in first]
+    bad = torch.zeros(len(first), dtype=torch.int32, device=first[0].device)
+    for _ in range(iters):
+        cur = fn()
+        assert len(cur) == len(first)
+        for j, (a, b) in enumerate(zip(cur, views)):
+            bad[j] += (a.detach().view(b.dtype) != b).any()
+    bad = bad.cpu().tolist()
+    assert not any(bad), {n: c for n, c in zip(names, bad) if c}

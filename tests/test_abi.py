@@ -22,7 +22,7 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), f"{name} declared in include/rgd_hip.h but not exported"
         assert name in _hip._SIGNATURES, f"{name} has no ctypes signature"
     assert sorted(_hip._SIGNATURES) == declared
-    assert lib.rgd_version() == 1000
+    assert lib.rgd_version() == 2000 and lib.rgd_version() // 1000 == _hip.ABI_MAJOR
     assert lib.rgd_attn_seqlen_q_rounded(1) == 64 and lib.rgd_attn_seqlen_q_rounded(128) == 128
     assert lib.rgd_attn_seqlen_q_rounded(129) == 192
     # delta (required part) plus room for the partial sums of split workgroups
@@ -45,9 +45,14 @@ def test_error_paths_return_codes_without_a_gpu():
     assert b"Only support fp16, bf16, and fp32" in lib.rgd_last_error()
     assert lib.rgd_rms_fwd(1, 1, 8, None, t3, t3, 0, 0, 1e-6, None) == -1
     assert lib.rgd_l2_fwd(70000, 1, 8, t3, t3, 0, 1e-6, None) == -1           # batch beyond the grid limit
-    # rows of any width stream through the forward; the backward (dw sums in registers) has a limit
-    assert lib.rgd_rms_bwd(1, 4, 200000, t3, t3, t3, t3, t3, 1, 0, 0, 1e-6, 0x1000, 1 << 30, None, 0, None) == -2
-    assert b"exceed the limit of the backward" in lib.rgd_last_error()
+    # the attention backward keeps offsets inside a staged tile in 32 bits: token strides of 2^24 elements are refused
+    far = _hip.Tensor4(0x1000, 64, 8, 1 << 24)
+    for pos in range(4):  # dout, q, k, v in turn
+        args = [t4] * 5
+        args[pos] = far
+        assert lib.rgd_attn_bwd(1, 1, 8, 8, 64, *args, 0x1000, None, 0, 0, t4, t4, t4, 1, 0, 0.125, 0x1000, 1 << 20,
+                                None) == -2, pos
+        assert b"token stride" in lib.rgd_last_error()
     assert lib.rgd_ln_qk_fwd(1, 1, 4, 4, 300, t4, t4, t4, t4, 0, 1e-6, None) == -1
     assert b"head dimensions up to 256" in lib.rgd_last_error()
     assert lib.rgd_rope_qk(1, 1, 4, 4, 160, t4, t4, t4, t4, 0x1000, 8, 32, 256, 32, 0, 4, 4, 0, 0, None) == -1
@@ -62,12 +67,10 @@ def test_error_paths_return_codes_without_a_gpu():
                             None) == -4
     # zero-sized problems are a successful no-op
     assert lib.rgd_l2_fwd(0, 0, 8, t3, t3, 0, 1e-6, None) == 0
-    ws, ct = ctypes.c_size_t(), ctypes.c_size_t()
-    assert lib.rgd_rms_bwd_workspace(4, 1024, 1024, 0, 0, ctypes.byref(ws), ctypes.byref(ct)) == 0
-    # one fp32 partial dw row per block; no counters are used (the argument stays in the interface)
-    assert ws.value >= 256 * 1024 * 4 and ct.value == 0
+    # one fp32 partial dw row per block
+    assert lib.rgd_rms_bwd_workspace(4, 1024, 1024, 0, 0) >= 256 * 1024 * 4
     # a too small workspace is refused before any launch
-    assert lib.rgd_rms_bwd(4, 1024, 1024, t3, t3, t3, t3, t3, 1, 0, 0, 1e-6, 0x1000, 16, 0x1000, 4, None) == -4
+    assert lib.rgd_rms_bwd(4, 1024, 1024, t3, t3, t3, t3, t3, 1, 0, 0, 1e-6, 0x1000, 16, None) == -4
 
 
 def test_module_api_surface_matches_reference():

@@ -3,7 +3,7 @@ tests/test_fused_rms.py (parity :139-211, seqdiff with different widths :213-328
 import pytest
 import torch
 
-from helpers import DTYPES, assert_close, gen, oracle, randn, to_gpu
+from helpers import DTYPES, assert_close, assert_repeats_bit_exact, gen, oracle, randn, to_gpu
 
 pytestmark = pytest.mark.gpu
 
@@ -99,21 +99,29 @@ def test_fused_rms_config5_and_module():
         FusedRMSNorm2(1536)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
-def test_fused_rms_deterministic(dtype):
+RACE_PAIRS = [(1, 239), (239, 1), (3, 799), (799, 3), (1024, 128), (97, 97), (128, 128), (200, 200), (256, 256),
+              (257, 257), (384, 384), (512, 512), (768, 768), (1024, 1024)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("unique_bw", [True, False])
+@pytest.mark.parametrize("C,dfactor", [(63, -0.75), (384, 0.6), (1023, 1.0)])
+@pytest.mark.parametrize("T1,T2", RACE_PAIRS)
+def test_fused_rms_norm_race_condition(T1, T2, C, dfactor, unique_bw, dtype):
+    """The reference's race test (tests/test_fused_rms.py:331-): batch 60, its 14 length pairs, 250 repeats, on three
+    of its nine widths and two of its five width ratios; every output and gradient must reproduce bit for bit."""
     from rgd_triton_amd import triton_fused_rms_func_fn
 
     g = gen(13)
-    x1, x2 = randn(g, 60, 113, 384, dtype=dtype), randn(g, 60, 203, 230, dtype=dtype)
-    w1, w2 = (1 + 0.1 * torch.randn(384, generator=g)).to(dtype), (1 + 0.1 * torch.randn(230, generator=g)).to(dtype)
-    d1, d2 = randn(g, 60, 113, 384, dtype=dtype).cuda(), randn(g, 60, 203, 230, dtype=dtype).cuda()
+    B, C2 = 60, max(1, int(C * (1 + dfactor)))
+    x1, x2 = randn(g, B, T1, C, dtype=dtype), randn(g, B, T2, C2, dtype=dtype)
+    w1 = (1 + 0.1 * torch.randn((B, 1, C) if unique_bw else (C,), generator=g)).to(dtype)
+    w2 = (1 + 0.1 * torch.randn((B, 1, C2) if unique_bw else (C2,), generator=g)).to(dtype)
+    d1, d2 = randn(g, B, T1, C, dtype=dtype).cuda(), randn(g, B, T2, C2, dtype=dtype).cuda()
     a = to_gpu(x1, x2, w1, w2, requires_grad=True)
-    first = None
-    for _ in range(25):
+
+    def step():
         y = triton_fused_rms_func_fn(*a)
-        gr = torch.autograd.grad(y, a, (d1, d2))
-        cur = [t.clone() for t in (*y, *gr)]
-        if first is None:
-            first = cur
-        else:
-            assert all(torch.equal(p, q) for p, q in zip(cur, first))
+        return (*y, *torch.autograd.grad(y, a, (d1, d2)))
+
+    assert_repeats_bit_exact(step, ("y1", "y2", "dx1", "dx2", "dw1", "dw2"))

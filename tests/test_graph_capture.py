@@ -33,9 +33,7 @@ class _Sequence:
                         bias=(0.3 * torch.randn(B, 1, T, T, generator=g)).to(dt).cuda())
         self.pe = oracle.rotary_table(T + 1, 32, 10000.0, dt).cuda()
         lib = self.lib
-        ws, ct = ctypes.c_size_t(), ctypes.c_size_t()
-        assert lib.rgd_rms_bwd_workspace(B, T, 384, 77, 640, ctypes.byref(ws), ctypes.byref(ct)) == 0
-        self.rms_ws = torch.empty(max(ws.value, 1), dtype=torch.uint8, device="cuda")
+        self.rms_ws = torch.empty(max(lib.rgd_rms_bwd_workspace(B, T, 384, 77, 640), 1), dtype=torch.uint8, device="cuda")
         self.attn_ws = torch.empty(lib.rgd_attn_bwd_workspace(B, H, T, T, D), dtype=torch.uint8, device="cuda")
         self.attn_fws = torch.empty(max(lib.rgd_attn_fwd_workspace(B, H, T, T, D), 16), dtype=torch.uint8, device="cuda")
         self.lse = torch.empty(B, H, lib.rgd_attn_seqlen_q_rounded(T), dtype=torch.float32, device="cuda")
@@ -63,7 +61,7 @@ class _Sequence:
         rc |= lib.rgd_fused_rms_bwd(B, T, 384, 77, 640, t3(i["d1"]), t3(i["x1"]), t3(i["w1"], 0), t3(out["dx1"]),
                                     t3(out["dw1"], 0), 1, t3(i["d2"]), t3(i["x2"]), t3(i["w2"], 0), t3(out["dx2"]),
                                     t3(out["dw2"], 0), 1, code, code, code, 1e-6, self.rms_ws.data_ptr(),
-                                    self.rms_ws.numel(), None, 0, st)
+                                    self.rms_ws.numel(), st)
         be = i["bias"].expand(B, H, T, T)
         bdesc = hip.Tensor4(be.data_ptr(), be.stride(0), be.stride(1), be.stride(2))
         scale = 1.0 / math.sqrt(D)

@@ -3,7 +3,7 @@ tests/test_head_layernorm.py, tests/test_head_rope.py and tests/test_fused_ln_ro
 import pytest
 import torch
 
-from helpers import DTYPES, assert_close, gen, oracle, randn, to_gpu
+from helpers import DTYPES, assert_close, assert_repeats_bit_exact, gen, oracle, randn, to_gpu
 
 pytestmark = pytest.mark.gpu
 
@@ -208,25 +208,51 @@ def test_ln_rope_config2_slice():
         assert_close(a, r, torch.bfloat16, "ln_rope", n)
 
 
-@pytest.mark.parametrize("which", ["ln", "rope", "ln_rope"])
-def test_head_ops_deterministic(which):
-    from rgd_triton_amd import triton_fused_ln_func_fn, triton_fused_ln_rope_fn, triton_rope_fn
+RACE_PAIRS = [(1, 239), (239, 1), (3, 799), (799, 3), (1024, 128), (97, 97), (128, 128), (200, 200), (256, 256),
+              (257, 257), (384, 384), (512, 512), (768, 768), (1024, 1024)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads_second", [True, False])
+@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("Tq,Tk", RACE_PAIRS)
+def test_head_ln_race_condition(Tq, Tk, D, heads_second, dtype):
+    """The reference's race test at its own strength (tests/test_head_layernorm.py:214-): batch 60, 4 heads, 250 repeats"""
+    from rgd_triton_amd import triton_fused_ln_func_fn
 
     g = gen(6)
-    q, k = _qk(g, 60, 4, 113, 203, 64, torch.float16, True)
-    gq, gk = _qk(g, 60, 4, 113, 203, 64, torch.float16, True)
-    pe = oracle.rotary_table(204, 32, dtype=torch.float16).to("cuda")
+    q, k = _qk(g, 60, 4, Tq, Tk, D, dtype, heads_second)
+    gq, gk = (t.cuda() for t in _qk(g, 60, 4, Tq, Tk, D, dtype, heads_second))
     qg, kg = to_gpu(q, k, requires_grad=True)
-    gq, gk = gq.cuda(), gk.cuda()
-    fn = {"ln": lambda: triton_fused_ln_func_fn(qg, kg, True),
-          "rope": lambda: triton_rope_fn(qg, kg, pe, (100, 150), True),
-          "ln_rope": lambda: triton_fused_ln_rope_fn(qg, kg, pe, (100, 150), True)}[which]
-    first = None
-    for _ in range(20):
+
+    def step():
+        out = triton_fused_ln_func_fn(qg, kg, heads_second)
+        return (*out, *torch.autograd.grad(out, (qg, kg), (gq, gk)))
+
+    assert_repeats_bit_exact(step, ("qo", "ko", "dq", "dk"))
+
+
+@pytest.mark.parametrize("which", ["rope", "ln_rope"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("heads_second", [True, False])
+@pytest.mark.parametrize("D,R", [(64, 32), (128, 96)])
+@pytest.mark.parametrize("Tq,Tk", RACE_PAIRS)
+def test_rope_race_condition(Tq, Tk, D, R, heads_second, dtype, which):
+    """The race tests of tests/test_head_rope.py and tests/test_fused_ln_rope.py: batch 60, their 14 length pairs, 250
+    repeats, on two of their (head dim, rotary dim) combinations; cutoffs inside both sequences."""
+    from rgd_triton_amd import triton_fused_ln_rope_fn, triton_rope_fn
+
+    g = gen(6)
+    q, k = _qk(g, 60, 4, Tq, Tk, D, dtype, heads_second)
+    gq, gk = (t.cuda() for t in _qk(g, 60, 4, Tq, Tk, D, dtype, heads_second))
+    pe = oracle.rotary_table(max(Tq, Tk) + 1, R, dtype=dtype).to("cuda")
+    qg, kg = to_gpu(q, k, requires_grad=True)
+    cut = (max(1, Tq * 3 // 4), max(1, Tk * 2 // 3))
+    fn = (lambda: triton_rope_fn(qg, kg, pe, cut, heads_second)) if which == "rope" else \
+        (lambda: triton_fused_ln_rope_fn(qg, kg, pe, cut, heads_second))
+
+    def step():
         out = fn()
-        gr = torch.autograd.grad(out, (qg, kg), (gq, gk))
-        cur = [t.clone() for t in (*out, *gr)]
-        if first is None:
-            first = cur
-        else:
-            assert all(torch.equal(a, b) for a, b in zip(cur, first))
+        return (*out, *torch.autograd.grad(out, (qg, kg), (gq, gk)))
+
+    assert_repeats_bit_exact(step, ("qo", "ko", "dq", "dk"))

@@ -40,12 +40,18 @@ def ref_head_norm(q, k, heads_second=False, eps=1e-6):
     return f(q), f(k)
 
 
-def ref_attention(q, k, v, bias=None):
+def ref_attention(q, k, v, bias=None, heads_per_chunk=4):
+    """fp32 attention in plain PyTorch, a few heads at a time (the scores of all 24 heads of the full-size joint block
+    would be 3.6 GB, several times over for autograd)"""
     d = q.shape[-1]
-    s = torch.einsum("bthd,bshd->bhts", q.float(), k.float()) / math.sqrt(d)
-    if bias is not None:
-        s = s + bias.float()
-    return torch.einsum("bhts,bshd->bthd", torch.softmax(s, -1), v.float()).to(q.dtype)
+    outs = []
+    for h0 in range(0, q.shape[2], heads_per_chunk):
+        hs = slice(h0, h0 + heads_per_chunk)
+        s = torch.einsum("bthd,bshd->bhts", q[:, :, hs].float(), k[:, :, hs].float()) / math.sqrt(d)
+        if bias is not None:
+            s = s + (bias if bias.shape[1] == 1 else bias[:, hs]).float()
+        outs.append(torch.einsum("bhts,bshd->bthd", torch.softmax(s, -1), v[:, :, hs].float()))
+    return torch.cat(outs, dim=2).to(q.dtype)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
@@ -79,14 +85,16 @@ def test_readme_attention_block(with_bias, dtype):
     assert torch.equal(blk(xa, bias), ya)
 
 
-def test_mmdit_joint_block_chain():
-    """BASELINE config 5 as a chain at reduced size (same structure: [image || text] joint sequence,
-    -inf bias on ~10 % of the text keys per batch element, everything bf16)."""
+@pytest.mark.parametrize("size", ["reduced", "config5"])
+def test_mmdit_joint_block_chain(size):
+    """BASELINE config 5 as a chain (the [image || text] joint sequence, -inf bias on ~10 % of the text keys per batch
+    element, everything bf16), at a reduced size and at its real size (2 x (4096 + 256) tokens, 1536 channels, 24 heads
+    of 64), forward and backward against the same chain in fp32 PyTorch on the CPU."""
     from rgd_triton_amd import FlashAttention, FusedHeadLayerNorm, FusedRMSNorm2
 
     g = gen(1005)
     dt = torch.bfloat16
-    B, Ti, Tt, C, H, D = 2, 640, 96, 384, 6, 64
+    B, Ti, Tt, C, H, D = (2, 640, 96, 384, 6, 64) if size == "reduced" else (2, 4096, 256, 1536, 24, 64)
     img, txt = randn(g, B, Ti, C, dtype=dt), randn(g, B, Tt, C, dtype=dt)
     w1 = (1 + 0.1 * torch.randn(C, generator=g)).to(dt)
     w2 = (1 + 0.1 * torch.randn(C, generator=g)).to(dt)

@@ -3,7 +3,7 @@ tests/test_l2normalize.py and tests/test_fused_l2normalize.py (inputs scaled x10
 import pytest
 import torch
 
-from helpers import DTYPES, assert_close, assert_close_allow_inf, gen, oracle, randn, to_gpu
+from helpers import DTYPES, assert_close, assert_close_allow_inf, assert_repeats_bit_exact, gen, oracle, randn, to_gpu
 
 pytestmark = pytest.mark.gpu
 
@@ -88,13 +88,29 @@ def test_fused_l2_module_and_determinism():
     x1, x2 = randn(g, 60, 113, 257, dtype=torch.float16, scale=100.0), randn(g, 60, 31, 64, dtype=torch.float16)
     d1, d2 = randn(g, 60, 113, 257, dtype=torch.float16).cuda(), randn(g, 60, 31, 64, dtype=torch.float16).cuda()
     x1g, x2g = to_gpu(x1, x2, requires_grad=True)
-    first = None
-    for _ in range(20):
+
+    def step():
         y = m(x1g, x2g)
-        gr = torch.autograd.grad(y, (x1g, x2g), (d1, d2))
-        cur = [t.clone() for t in (*y, *gr)]
-        if first is None:
-            first = cur
-        else:
-            assert all(torch.equal(p, q) for p, q in zip(cur, first))
+        return (*y, *torch.autograd.grad(y, (x1g, x2g), (d1, d2)))
+
+    assert_repeats_bit_exact(step, ("y1", "y2", "dx1", "dx2"))
     assert m.cache.fwd is not None and m.cache.bwd is not None
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("C", [32, 63, 97, 122, 257, 384, 510, 740, 1023])
+@pytest.mark.parametrize("T", [14, 128, 1024])
+def test_l2_norm_race_condition(T, C, dtype):
+    """The race test of tests/test_l2normalize.py: batch 60, its 9 widths, 250 repeats (three of its eight lengths)"""
+    from rgd_triton_amd import triton_norm_func_fn
+
+    g = gen(4)
+    x = randn(g, 60, T, C, dtype=dtype)
+    dy = randn(g, 60, T, C, dtype=dtype).cuda()
+    xg = to_gpu(x, requires_grad=True)
+
+    def step():
+        y = triton_norm_func_fn(xg)
+        return (y, *torch.autograd.grad(y, (xg,), dy))
+
+    assert_repeats_bit_exact(step, ("y", "dx"))

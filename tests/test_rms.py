@@ -3,7 +3,7 @@ Counterpart of the reference's tests/test_rms.py (parity :126-184, race :188-246
 import pytest
 import torch
 
-from helpers import DTYPES, assert_close, gen, oracle, randn, to_gpu
+from helpers import DTYPES, assert_close, assert_repeats_bit_exact, gen, oracle, randn, to_gpu
 
 pytestmark = pytest.mark.gpu
 
@@ -55,23 +55,13 @@ def test_rms_norm_wide_rows(T, unique_bw, C, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("C,unique_bw", [(8200, False), (10001, False), (12288, True), (16384, False)])
+@pytest.mark.parametrize("C,unique_bw", [(8200, False), (10001, False), (12288, True), (16384, False), (20000, False),
+                                         (20001, True), (32768, True), (65536, False), (70003, False)])
 def test_rms_norm_streamed_rows(C, unique_bw, dtype):
-    """Rows beyond the register-resident limit take the two-pass streaming kernel (the reference loops over
-    channel blocks for any C); its backward holds the dw sums of 16384 channels (8192 unaligned) at most."""
-    from rgd_triton_amd import triton_rms_func_fn
-
+    """Rows beyond the register-resident limit take the two-pass streaming kernel, at any width like the reference
+    (it loops over channel blocks, rmsnorm_cached.py:198-219): the dw sums of the backward stay in registers one
+    slab of 16384 channels (8192 on the unaligned path) at a time."""
     B, T = 2, 37
-    if C % 8 and C > 8192:  # odd width: forward only, the backward must refuse
-        g = gen(C)
-        x = randn(g, B, T, C, dtype=dtype)
-        w = (1 + 0.1 * torch.randn(C, generator=g)).to(dtype)
-        xg, wg = to_gpu(x, w, requires_grad=True)
-        y = triton_rms_func_fn(xg, wg, 1e-6)
-        assert_close(y, oracle.rms_fwd(x, w, 1e-6), dtype, "rms", "y")
-        with pytest.raises(RuntimeError, match="exceed the limit of the backward"):
-            torch.autograd.grad(y, (xg, wg), torch.ones_like(y))
-        return
     (y, dx, dw), (y_ref, dx_ref, dw_ref) = _run(B, T, C, dtype, unique_bw, seed=C)
     assert_close(y, y_ref, dtype, "rms", "y")
     assert_close(dx, dx_ref, dtype, "rms", "dx")
@@ -126,29 +116,39 @@ def test_rms_strided_views():
     assert_close(dw, dw_ref, torch.float16, "rms", "dw", atol_scale=3 * 100 * 16)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("unique_bw", [True, False])
+@pytest.mark.parametrize("C", [32, 63, 97, 122, 257, 384, 510, 740, 1023])
+@pytest.mark.parametrize("T", [14, 31, 97, 128, 200, 384, 768, 1024])
+def test_rms_norm_race_condition(T, C, unique_bw, dtype):
+    """The reference's race test at its own strength (tests/test_rms.py:187-246): batch 60, its 9 widths x 8 lengths x
+    both weight forms x 3 dtypes, 250 repeats.  The reference allows dx and dw to move by rounding noise; here y, dx
+    and dw must reproduce bit for bit."""
+    _race(60, T, C, dtype, unique_bw)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("C,T", [(384, 239), (1023, 113), (1536, 512), (6144, 67), (12288, 19)])
-def test_rms_deterministic(C, T, dtype):
-    """The reference's race test (tests/test_rms.py:193-246): batch 60, repeated runs must give
-    bit-identical y, dx and dw."""
+@pytest.mark.parametrize("C,T", [(1536, 512), (6144, 67), (12288, 19), (40000, 5)])
+def test_rms_deterministic_wide(C, T, dtype):
+    """the same loop on the multi-wavefront and streaming kernels (widths the reference's tests do not reach)"""
+    _race(60 if C < 40000 else 12, T, C, dtype, False)
+
+
+def _race(B, T, C, dtype, unique_bw):
     from rgd_triton_amd import triton_rms_func_fn
 
     g = gen(7)
-    x = randn(g, 60, T, C, dtype=dtype)
-    w = (1 + 0.1 * torch.randn(C, generator=g)).to(dtype)
-    dy = randn(g, 60, T, C, dtype=dtype)
+    x = randn(g, B, T, C, dtype=dtype, shift=0.5)
+    w = (1 + 0.1 * torch.randn((B, 1, C) if unique_bw else (C,), generator=g)).to(dtype)
+    dy = randn(g, B, T, C, dtype=dtype)
     xg, wg = to_gpu(x, w, requires_grad=True)
     dyg = dy.to("cuda")
-    first = None
-    for _ in range(25):
+
+    def step():
         y = triton_rms_func_fn(xg, wg, 1e-6)
-        dx, dw = torch.autograd.grad(y, (xg, wg), dyg)
-        cur = (y.clone(), dx.clone(), dw.clone())
-        if first is None:
-            first = cur
-        else:
-            for a, b, n in zip(cur, first, ("y", "dx", "dw")):
-                assert torch.equal(a, b), f"{n} differs between runs"
+        return (y, *torch.autograd.grad(y, (xg, wg), dyg))
+
+    assert_repeats_bit_exact(step, ("y", "dx", "dw"))
 
 
 def test_module_state_dict_and_cache():
