@@ -29,14 +29,24 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16/fp16
+BWD_KERNELS = "attn_bwd_dq_kernel + attn_bwd_dkv_kernel (one rgd_attn_bwd call)"
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# this file (profiles/), scaled by a copy kernel of known size; None until measured for a workload.
-MEASURED_TRAFFIC = {
-    # FETCH_SIZE 65737.6 KiB x 2.0 (copy calibration) + WRITE_SIZE 65536.0 KiB x 1.0, per launch of the
-    # LN+RoPE backward on this workload (profiles/head_rows_lnrope_config2.md)
-    "ln_rope_bwd_c2": 201739469,
-}
+PROFILE_SUMMARY = os.path.join("profiles", "head_rows_lnrope_config2.md")
+
+
+def profile_figures(path=PROFILE_SUMMARY):
+    """Figures of the dominant kernel that only a profiler run can give (HBM traffic counters, the kernel-trace
+    duration), read from the committed rocprofv3 summary: lines `bench.<key> = <value>` at its end, next to the
+    commit they were measured at.  Nothing is reported when the file or a key is missing."""
+    out = {}
+    try:
+        for line in open(os.path.join(ROOT, path)):
+            if line.startswith("bench.") and "=" in line:
+                k, v = line[len("bench."):].split("=", 1)
+                out[k.strip()] = v.strip()
+    except OSError:
+        pass
+    return out
 
 
 def parse():
@@ -63,6 +73,8 @@ def timed_loop(torch, step_fns, steps, warmup):
     [fwd, bwd] given an event recorder.  Returns (wall ms per step, event span ms per step, fwd ms list,
     bwd ms list, event-to-event gap ms)."""
     n = len(step_fns)
+    # untimed: bring the clocks to their steady state whatever --warmup says, then the W warm-up steps
+    spin_up(torch, lambda i: step_fns[i % n](None), 0.1)
     for i in range(warmup):
         step_fns[i % n](None)
     # timed region: exactly `steps` steps between two synchronisations; only the two bracketing events
@@ -351,7 +363,15 @@ def attention_case(torch, name, B, T, H, D, dtype, bias_kind, iters=20, with_cpu
     bias_gbs = None if bias is None else round(3.0 * B * H * T * T * bias.element_size() / tot / 1e6, 1)
     cpu = cpu_extra(torch, "attention", B=B, T=T, H=H, D=D, dtype=dtype, bias=bias) if with_cpu else None
     sdpa = torch_sdpa_case(torch, q, k, v, do, bias, flops) if with_cpu else None
-    return {"workload": name, "cpu_baseline": cpu, "torch_sdpa": sdpa, "bias_read_gbs": bias_gbs, "fwd_ms": round(f_ms, 4), "bwd_ms": round(b_ms, 4),
+    # roofline of the slower of the two calls (MFMA-bound; algorithmic FLOPs 4/14 forward, 10/14 backward)
+    f_tf, b_tf = flops * 4 / 14 / f_ms / 1e9, flops * 10 / 14 / b_ms / 1e9
+    slow_bwd = b_tf <= f_tf
+    roof = {"bound": "mfma", "kernel": BWD_KERNELS if slow_bwd else "attn_fwd_kernel (rgd_attn_fwd)",
+            "achieved": round(b_tf if slow_bwd else f_tf, 2), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": round((b_tf if slow_bwd else f_tf) / MFMA_PEAK_TFLOPS, 4),
+            "avg_launch_ms": round(b_ms if slow_bwd else f_ms, 4),
+            "duration_source": "HIP events around the call, mean of %d" % iters}
+    return {"workload": name, "roofline": roof, "cpu_baseline": cpu, "torch_sdpa": sdpa, "bias_read_gbs": bias_gbs, "fwd_ms": round(f_ms, 4), "bwd_ms": round(b_ms, 4),
             "tflops": round(flops / tot / 1e9, 2), "fwd_tflops": round(flops * 4 / 14 / f_ms / 1e9, 2),
             "bwd_tflops": round(flops * 10 / 14 / b_ms / 1e9, 2), "frac_mfma_peak": round(flops / tot / 1e9 / MFMA_PEAK_TFLOPS, 4)}
 
@@ -558,6 +578,9 @@ def main():
     ms = max(wall_ms, gpu_ms)
     bwd_avg, fwd_avg = statistics.mean(bwd), statistics.mean(fwd)
     achieved = bwd_bytes / bwd_avg / 1e6
+    prof = profile_figures()
+    traffic = int(prof["traffic_bytes_per_launch"]) if "traffic_bytes_per_launch" in prof else None
+    rocprof_us = float(prof["rocprof_avg_launch_us"]) if "rocprof_avg_launch_us" in prof else None
     result = {
         "metric": "attn fwd+bwd TFLOP/s (% MFMA peak); norm/RoPE GB/s (% HBM peak)",
         "value": round(step_bytes / ms / 1e6, 1),
@@ -571,9 +594,16 @@ def main():
                    "algorithmic_bytes_per_step": step_bytes},
         "roofline": {"bound": "hbm", "kernel": "head_rows_kernel<bf16, LNROPE_BWD> (rgd_ln_rope_qk_bwd)",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get("ln_rope_bwd_c2"),
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                      "algorithmic_bytes_per_launch": bwd_bytes, "avg_launch_ms": round(bwd_avg, 5),
+                     "duration_source": "HIP events recorded around every launch of the timed steps (a second pass over "
+                                        "the same steps), minus the event-to-event cost measured in that pass",
                      "event_gap_ms_subtracted": round(event_gap, 5),
+                     # not measured by this run: the committed rocprofv3 summary of this same command
+                     "from_profile": {"file": PROFILE_SUMMARY, "measured_at": prof.get("measured_at"),
+                                      "traffic_bytes_per_launch": traffic, "rocprof_avg_launch_us": rocprof_us,
+                                      "frac_at_rocprof_duration": None if not rocprof_us else
+                                      round(bwd_bytes / rocprof_us / 1e3 / HBM_PEAK_GBS, 4)},
                      "fwd_kernel": {"achieved": round(fwd_bytes / fwd_avg / 1e6, 1), "avg_launch_ms": round(fwd_avg, 5),
                                     "frac": round(fwd_bytes / fwd_avg / 1e6 / HBM_PEAK_GBS, 4)}},
         "timing": {"wall_ms_per_step": round(wall_ms, 5), "gpu_event_span_ms_per_step": round(gpu_ms, 5)},

@@ -52,6 +52,17 @@ def _seen(cache, field, key):
     return False
 
 
+def _no_capture(what):
+    """Every backward starts here.  Recording an autograd backward of these operators into a HIP graph ended in a
+    crash inside the runtime's end-of-capture call on the one occasion it was tried (the backward nodes run on
+    autograd's worker thread), and its cause was never established, so the combination is refused with an error
+    instead: record the backward through direct C-ABI calls (tests/test_graph_capture.py does) or keep autograd
+    outside the graph.  The forward functions can be captured."""
+    if torch.cuda.is_current_stream_capturing():
+        raise RuntimeError(f"{what}: an autograd backward cannot be recorded into a HIP graph with this package; "
+                           "record direct calls of the C ABI instead")
+
+
 def _sig(*ts):
     return tuple((tuple(t.shape), t.dtype, tuple(t.stride())) if t is not None else None for t in ts)
 
@@ -107,6 +118,7 @@ class RMS_Func(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dy):
+        _no_capture("RMS_Func.backward")
         (dy,) = _lastdim_contig(dy)
         x, w = ctx.saved_tensors
         shared, w_sb = ctx.w_layout
@@ -156,6 +168,7 @@ class Fused_RMS_Func(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dy1, dy2):
+        _no_capture("Fused_RMS_Func.backward")
         dy1, dy2 = _lastdim_contig(dy1, dy2)
         x1, x2, w1, w2 = ctx.saved_tensors
         (s1, sb1), (s2, sb2) = ctx.layouts
@@ -208,6 +221,7 @@ class Norm_Func(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dy):
+        _no_capture("Norm_Func.backward")
         (dy,) = _lastdim_contig(dy)
         (x,) = ctx.saved_tensors
         B, T, C = x.shape
@@ -247,6 +261,7 @@ class Fused_Norm_Func(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dy1, dy2):
+        _no_capture("Fused_Norm_Func.backward")
         dy1, dy2 = _lastdim_contig(dy1, dy2)
         x1, x2 = ctx.saved_tensors
         B, T1, C1 = x1.shape
@@ -333,6 +348,7 @@ class Fused_LNQK_Func(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, doq, dok):
+        _no_capture("Fused_LNQK_Func.backward")
         q, k = ctx.saved_tensors
         hs = ctx.heads_second
         doq, dok = _lastdim_contig(doq, dok)
@@ -378,6 +394,7 @@ class CombinedRoPEFunc(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, doq, dok):
+        _no_capture("CombinedRoPEFunc.backward")
         (pos_emb,) = ctx.saved_tensors
         assert not ctx.needs_input_grad[2], "CombinedRoPE does not support gradients in position embeddings"
         hs = ctx.heads_second
@@ -425,6 +442,7 @@ class FusedRoPEFunc(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, doq, dok):
+        _no_capture("FusedRoPEFunc.backward")
         q, k, pos_emb = ctx.saved_tensors
         assert not ctx.needs_input_grad[2], "CombinedRoPE does not support gradients in position embeddings"
         hs = ctx.heads_second
@@ -540,6 +558,7 @@ class FlashAttnFunc(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, do, dlse):
+        _no_capture("FlashAttnFunc.backward")
         q, k, v, o, lse, bias = ctx.saved_tensors
         assert not ctx.needs_input_grad[3], "FlashAttention does not support bias gradient yet"
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)

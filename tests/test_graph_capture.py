@@ -96,3 +96,30 @@ def test_c_abi_sequence_replays_from_a_graph():
         for name, t in graph_out.items():
             assert not torch.isnan(t.float()).any(), f"replay {rep}: {name} holds NaN"
             assert torch.equal(t, eager_out[name]), f"replay {rep}: {name} differs from the eager run"
+
+
+@pytest.mark.skip(reason="recording an autograd backward into a HIP graph aborted inside the runtime's end-of-capture "
+                         "call when it was first tried; no output of that run was kept and reading the code has not "
+                         "shown a cause, so the case stays off the GPU and the package refuses it with an error "
+                         "(functional._no_capture)")
+def test_autograd_forward_backward_replays_from_a_graph():
+    """What the case would be: the Module API, forward and backward through autograd, recorded and replayed."""
+    from rgd_triton_amd import FlashAttention
+
+    g = gen(32)
+    q, k, v, do = (randn(g, 2, 300, 4, 64, dtype=torch.bfloat16).cuda() for _ in range(4))
+    q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
+    attn = FlashAttention()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):  # warm-up off the default stream, as torch's graph recipe asks
+        torch.autograd.grad(attn(q, k, v), (q, k, v), do)
+    torch.cuda.current_stream().wait_stream(side)
+    eager = torch.autograd.grad(attn(q, k, v), (q, k, v), do)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = torch.autograd.grad(attn(q, k, v), (q, k, v), do)
+    for _ in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(captured, eager):
+            assert torch.equal(a, b)

@@ -1,5 +1,6 @@
-"""Calls on side streams: every operator launches on torch's current stream and keeps its scratch per stream, so two
-streams that run different problems at the same time give, bit for bit, what each gives alone on the default stream."""
+"""Calls on side streams: every operator launches on torch's current stream and takes its scratch per call from the
+caching allocator (which never hands a block to another stream while it is in use), so two streams that run different
+problems at the same time give, bit for bit, what each gives alone on the default stream."""
 import pytest
 import torch
 
