@@ -99,6 +99,20 @@ int rgd_rms_bwd(int64_t B, int64_t T, int64_t C,
                 int x_dtype, int w_dtype, float eps,
                 void* workspace, size_t workspace_bytes, void* stream);
 
+/* rgd_rms_bwd for callers that cannot allocate device memory and have no workspace to hand over (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+ * Same arguments, kernels and results (bit for bit) as rgd_rms_bwd, minus the workspace: the partial dw rows live
+ * in a device array that is part of the library's code object (rgd_rms_bwd_noalloc_limit() bytes, 16 MiB, per GPU,
+ * held until the process ends).  The call makes no hipMalloc / hipFree and uses no allocating routine.  Shapes
+ * whose rgd_rms_bwd_workspace(B, T, C, 0, 0) exceeds the limit are refused with RGD_ERR_WORKSPACE.
+ * All calls on one GPU share that array: calls that may overlap in time on one GPU (different streams or
+ * threads) race on it; callers that need overlap use rgd_rms_bwd with a workspace each. */
+size_t rgd_rms_bwd_noalloc_limit(void);
+int rgd_rms_bwd_noalloc(int64_t B, int64_t T, int64_t C,
+                        const rgd_tensor3* dy, const rgd_tensor3* x, const rgd_tensor3* w,
+                        const rgd_tensor3* dx, const rgd_tensor3* dw, int w_shared,
+                        int x_dtype, int w_dtype, float eps, void* stream);
+
 /* replaces _fused_rms_fwd, normalization/fused_rmsnorm_cached.py:389-501 (kernel :6-125):
  * the two tensors are normalised in one launch as one virtual tensor; they share B and the dtype,
  * and have independent T, C and weights. */

@@ -42,6 +42,8 @@ _SIGNATURES = {
     "rgd_rms_fwd": (_int, [_i64, _i64, _i64, _T3, _T3, _T3, _int, _int, _f32, _vp]),
     "rgd_rms_bwd_workspace": (_sz, [_i64] * 5),
     "rgd_rms_bwd": (_int, [_i64, _i64, _i64, _T3, _T3, _T3, _T3, _T3, _int, _int, _int, _f32, _vp, _sz, _vp]),
+    "rgd_rms_bwd_noalloc_limit": (_sz, []),
+    "rgd_rms_bwd_noalloc": (_int, [_i64, _i64, _i64, _T3, _T3, _T3, _T3, _T3, _int, _int, _int, _f32, _vp]),
     "rgd_fused_rms_fwd": (_int, [_i64] * 5 + [_T3] * 6 + [_int, _int, _int, _f32, _vp]),
     "rgd_fused_rms_bwd": (_int, [_i64] * 5 + [_T3] * 5 + [_int] + [_T3] * 5 + [_int] + [_int, _int, _int, _f32,
                                                                                  _vp, _sz, _vp]),

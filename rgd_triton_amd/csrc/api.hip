@@ -6,6 +6,8 @@
 
 // attn_f16.hip / attn_bf16.hip: LDS size attribute of every attention kernel instantiation of one element type
 template <typename T> int attn_configure_all();
+// rows_wide.hip: address of the library-owned scratch array on the current device
+int wide_noalloc_setup(void** out);
 
 namespace {
 thread_local char g_error[512] = "";
@@ -22,6 +24,7 @@ void init_once() {
         // kernels with more than 48 KB of dynamic LDS need the attribute before their first launch
         rc = attn_configure_all<f16_t>();
         if (rc == RGD_OK) rc = attn_configure_all<bf16_t>();
+        if (rc == RGD_OK) rc = wide_noalloc_setup(nullptr);
     } else {
         // no usable device (a CPU-only process that checks arguments): launches will fail with their own error
         (void)hipGetLastError();

@@ -398,6 +398,11 @@ struct WideHalfArgs {
 int wide_launch(const char* name, int op, bool bwd, int64_t B, const WideHalfArgs& a1, const WideHalfArgs& a2,
                 int dtype, float eps, void* workspace, size_t workspace_bytes, void* stream);
 size_t wide_workspace(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2);
+// bytes of the library-owned scratch array behind rgd_rms_bwd_noalloc (one copy per GPU, held for the process' life)
+#ifndef RGD_NOALLOC_SCRATCH_BYTES
+#define RGD_NOALLOC_SCRATCH_BYTES (16u << 20)
+#endif
+int wide_noalloc_setup(void** out);  // rows_wide.hip: address of that array on the current device
 
 // per-dtype instantiation units (rows_wide_f32.hip, rows_wide_f16.hip, rows_wide_bf16.hip)
 struct WideConfig {

@@ -3,6 +3,8 @@
 #include "rows_wide.h"
 
 #include <algorithm>
+#include <atomic>
+#include <mutex>
 #include <string.h>
 
 #ifndef RGD_DW_BLOCKS_PER_CU
@@ -233,6 +235,48 @@ int wide_launch(const char* name, int op, bool bwd, int64_t B, const WideHalfArg
 }
 
 // ------------------------------------------------------------------------------------------
+// Scratch owned by the library, for the entry point that must not allocate (rgd_rms_bwd_noalloc): the partial dw
+// rows live in this file-scope device array instead of a caller's workspace.  Every GPU the library runs on holds
+// its own copy of the array, at its own address, until the process ends.  In host code the array's name is only a
+// handle for hipGetSymbolAddress; the address that call returns for a device is what kernels and runtime calls get.
+// ------------------------------------------------------------------------------------------
+constexpr size_t kNoAllocScratchBytes = RGD_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+std::mutex g_scratch_mutex;
+}  // namespace
+
+// Resolves the scratch array's address on the CURRENT device (once per device); *out receives it.
+int wide_noalloc_setup(void** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        rgd_set_error("rgd_rms_bwd_noalloc: no current device (or a device index of %d or more)", kMaxDevices);
+        return RGD_ERR_INVALID;
+    }
+    void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        ptr = g_scratch_ptr[dev].load(std::memory_order_relaxed);
+        if (!ptr) {
+            const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+            if (e != hipSuccess || !ptr) {
+                (void)hipGetLastError();
+                rgd_set_error("rgd_rms_bwd_noalloc: hipGetSymbolAddress(scratch) failed on device %d: %s", dev,
+                              hipGetErrorString(e));
+                return RGD_ERR_LAUNCH;
+            }
+            g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+        }
+    }
+    if (out) *out = ptr;
+    return RGD_OK;
+}
+
+// ------------------------------------------------------------------------------------------
 // C ABI
 // ------------------------------------------------------------------------------------------
 namespace {
@@ -271,6 +315,29 @@ int rgd_rms_bwd(int64_t B, int64_t T, int64_t C, const rgd_tensor3* dy, const rg
                 void* workspace, size_t workspace_bytes, void* stream) {
     return wide_launch("rgd_rms_bwd", WIDE_RMS, true, B, half(T, C, x, dy, dx, w, dw, w_dtype, w_shared), kNoHalf,
                        x_dtype, eps, workspace, workspace_bytes, stream);
+}
+
+size_t rgd_rms_bwd_noalloc_limit(void) { return kNoAllocScratchBytes; }
+
+int rgd_rms_bwd_noalloc(int64_t B, int64_t T, int64_t C, const rgd_tensor3* dy, const rgd_tensor3* x,
+                        const rgd_tensor3* w, const rgd_tensor3* dx, const rgd_tensor3* dw, int w_shared, int x_dtype,
+                        int w_dtype, float eps, void* stream) {
+    const char* name = "rgd_rms_bwd_noalloc";
+    const int init_rc = rgd_ensure_init();
+    if (init_rc != RGD_OK) return init_rc;
+    // the size rgd_rms_bwd_workspace asks a caller for must fit the fixed array
+    RGD_REQUIRE(B >= 0 && T >= 0 && C >= 0, RGD_ERR_INVALID, "%s: negative shape", name);
+    const size_t need = wide_workspace(B, T, C, 0, 0);
+    RGD_REQUIRE(need <= kNoAllocScratchBytes, RGD_ERR_WORKSPACE,
+                "%s: (B=%lld, T=%lld, C=%lld) needs %zu bytes of scratch, the library's fixed scratch holds %zu; use "
+                "rgd_rms_bwd with a workspace", name, (long long)B, (long long)T, (long long)C, need,
+                kNoAllocScratchBytes);
+    void* ptr = nullptr;
+    const int rc = wide_noalloc_setup(&ptr);  // one atomic load once the device has been seen
+    if (rc != RGD_OK) return rc;
+    // every partial row the reduce kernel reads is written by this call's first kernel: nothing has to start at 0
+    return wide_launch(name, WIDE_RMS, true, B, half(T, C, x, dy, dx, w, dw, w_dtype, w_shared), kNoHalf, x_dtype, eps,
+                       ptr, kNoAllocScratchBytes, stream);
 }
 
 int rgd_fused_rms_fwd(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2, const rgd_tensor3* x1,
