@@ -21,6 +21,8 @@
 
 #include "attn_common.h"
 
+#include <type_traits>
+
 constexpr int BWD_THREADS = 256;
 constexpr int BWD_BM = 128;  // rows (queries or keys) owned by a workgroup
 
@@ -266,8 +268,6 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
             if constexpr (HAS_BIAS)
                 bias_nxt.load(bias_row, key0 + BN, g, p.Tk, F || (p.bias_vec && key0 + 2 * BN <= p.Tk));
         }
-        float bias_v[NKB][16];
-        if constexpr (HAS_BIAS) bias_cur.decode(bias_v);
         const T* ks = ks_base + buf * TILE + a_off;
         const T* vs = vs_base + buf * TILE + a_off;
         // the dP accumulators start from -delta, so that product comes out as dP - delta
@@ -290,6 +290,14 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
                 dp[kb] = MM::run(as_v8<T>(va), doreg[c], dp[kb]);
             }
         }
+        // A tile whose bias is -inf for every (query, key) pair of this wavefront has P = 0 and dS = 0: the rest of
+        // the step is left out.  Tested where the bias is first needed, after the first two products have been
+        // issued, so the bias loads keep the time of those products to arrive.
+        bool masked_tile = false;
+        if constexpr (attn_skip_masked(DPAD, BIAS)) masked_tile = bias_cur.all_neg_inf(0, NKB);
+        if (!masked_tile) {
+        float bias_v[NKB][16];
+        if constexpr (HAS_BIAS) bias_cur.decode(bias_v);
         // t = logit - lse (log2 domain)
 #pragma unroll
         for (int kb = 0; kb < NKB; ++kb)
@@ -338,6 +346,7 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
                 acc[d] = MM::run(as_v8<T>(a), bop, acc[d]);
             }
         }
+        }  // !masked_tile
         if (F || j + 1 < t_end) {
             store_tiles(buf ^ 1, IntC<(AH == 0 ? 0 : 2 - AH)>{});
             if constexpr (HAS_BIAS) bias_cur = bias_nxt;
@@ -448,6 +457,17 @@ template <typename TB> struct BiasColumn {
 #pragma unroll
         for (int v = 0; v < 16; ++v) out[v] = static_cast<float>(raw[v]);
     }
+    // per lane: every one of the 16 values is -inf (the caller combines lanes and sub-tiles)
+    __device__ __forceinline__ bool first_is_neg_inf() const { return bits(0) == NEG_INF; }
+    __device__ __forceinline__ bool lane_all_neg_inf() const {
+        bool all = true;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) all = all && bits(v) == NEG_INF;
+        return all;
+    }
+    typedef typename std::conditional<sizeof(TB) == 2, uint16_t, uint32_t>::type Bits;
+    static constexpr Bits NEG_INF = (Bits)(NegInfBits<TB>::value & (sizeof(TB) == 2 ? 0xFFFFu : 0xFFFFFFFFu));
+    __device__ __forceinline__ Bits bits(int v) const { return __builtin_bit_cast(Bits, raw[v]); }
 };
 
 template <typename T, int DPAD, int BIAS>
@@ -680,6 +700,22 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_D
                     dp[u] = MM::run(as_v8<T>(da), vreg[c], dp[u]);
                 }
         }
+        // a step whose bias is -inf for every (query, key) pair of this wavefront has P = 0 and dS = 0: the rest of the step
+        // is left out (tested where the bias is first needed, after the first two products have been issued).
+        // The first value of every lane is looked at first, so a step with ordinary values costs a few instructions.
+        bool masked_step = false;
+        if constexpr (attn_skip_masked(DPAD, BIAS)) {
+            bool first = true;
+#pragma unroll
+            for (int u = 0; u < NSUB; ++u) first = first && b_use[u].first_is_neg_inf();
+            if (__builtin_amdgcn_ballot_w64(!first) == 0) {
+                bool all = true;
+#pragma unroll
+                for (int u = 0; u < NSUB; ++u) all = all && b_use[u].lane_all_neg_inf();
+                masked_step = __builtin_amdgcn_ballot_w64(!all) == 0;
+            }
+        }
+        if (!masked_step) {
 #pragma unroll
         for (int u = 0; u < NSUB; ++u) {
             const int q0 = j * BQ + u * 32;
@@ -766,6 +802,7 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_D
                 }
             }
         }
+        }  // !masked_step
         if (F || j + 1 < ntiles) {
             store_tiles(buf ^ 1);
             if constexpr (HAS_BIAS && PP == 2) {

@@ -245,6 +245,8 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
         }
         if constexpr (!SPLIT_HALVES) {
             // d <= 64: both 32-key halves of the tile go through the softmax together
+            // A tile whose bias is -inf for every (query, key) pair of this wavefront adds nothing (p = 0 exactly):
+            // its products and its softmax are left out.
 
             // ---- S^T = K . Q^T ----
             const T* ks = ks_base + buf * TILE + a_off;
@@ -262,6 +264,12 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
                     s[kb] = MM::run(as_v8<T>(a), qreg[c], s[kb]);
                 }
 
+            // A tile whose bias is -inf for every (query, key) pair of this wavefront adds nothing (p = 0 exactly):
+            // its softmax and its second product are left out.  The test sits where the bias is first needed, after
+            // the first product has been issued, so the bias loads keep the time of that product to arrive.
+            bool masked_tile = false;
+            if constexpr (attn_skip_masked(DPAD, BIAS)) masked_tile = bias_cur.all_neg_inf(0, 2);
+            if (!masked_tile) {
             // ---- t = logit - m_ref (log2 domain) ----
             const float m_off = m_ref == -INFINITY ? 0.f : m_ref;
 #pragma unroll
@@ -369,6 +377,7 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
                     oacc[d] = MM::run(as_v8<T>(a), pb, oacc[d]);
                 }
             }
+            }  // !masked_tile
         } else {
             // Each 32-key half of the tile is a complete softmax step of its own (S -> p -> PV), so only 16
             // logits are live at a time; the register budget buys wavefronts per SIMD, and those hide the
@@ -386,6 +395,11 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
                 for (int c = 0; c < NC; ++c) {
                     const u32x4 a = *reinterpret_cast<const u32x4*>(ks + kb * 32 * ST + c * 16);
                     s = MM::run(as_v8<T>(a), qreg[c], s);
+                }
+                // a half whose bias is -inf everywhere for this wavefront adds nothing: its softmax and second
+                // product are left out (tested where the bias is first needed, see above)
+                if constexpr (attn_skip_masked(DPAD, BIAS)) {
+                    if (bias_cur.all_neg_inf(kb, 1)) continue;
                 }
 
                 // ---- t = logit - m_ref (log2 domain) ----

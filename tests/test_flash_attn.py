@@ -268,6 +268,37 @@ def test_flash_attn_masked_bias_no_nan():
     check(got, reference(qb, kb, vb, first.to(torch.bfloat16), dob), T, grad_mult=3, name="first tile masked")
 
 
+@pytest.mark.parametrize("dtype", HALF)
+@pytest.mark.parametrize("bias_dtype", ["same", "fp32"])
+@pytest.mark.parametrize("d", [32, 64, 128])
+@pytest.mark.parametrize("block", [32, 64, 128, 96])
+def test_flash_attn_masked_tiles(block, d, bias_dtype, dtype):
+    """Blocks of -inf in the bias whose edges sit on, and off, the kernels' tile edges: the kernels leave out a block of
+    logits when every bias value a wavefront holds for it is -inf, and the result must be what the full computation
+    gives (block-diagonal + random visible blocks; ragged lengths so the last tiles are partial; one batch element has
+    a (B,1,Q,K) broadcast row of NaN-free ordinary values so unmasked tiles sit next to masked ones)."""
+    g = gen(9)
+    B, H, Tq, Tk = 2, 3, 330, 420
+    q, k, v = randn(g, B, Tq, H, d, dtype=dtype), randn(g, B, Tk, H, d, dtype=dtype), randn(g, B, Tk, H, d, dtype=dtype)
+    do = randn(g, B, Tq, H, d, dtype=dtype)
+    bt = torch.float32 if bias_dtype == "fp32" else dtype
+    bias = (0.5 * torch.randn(B, H, Tq, Tk, generator=g))
+    qi, ki = torch.arange(Tq) // block, torch.arange(Tk) // block
+    visible = torch.rand(B, H, qi.max() + 1, ki.max() + 1, generator=g) < 0.4
+    visible[..., 0] = True  # every query row keeps its first key block
+    mask = ~visible[:, :, qi][:, :, :, ki]
+    bias = bias.masked_fill(mask, float("-inf")).to(bt)
+    ref = reference(q, k, v, bias, do)
+    if bias_dtype == "fp32":  # the low-precision comparison run adds the bias in q's dtype
+        ref = ref[:3] + reference(q, k, v, bias.to(dtype), do)[3:]
+    got = run_case(q, k, v, bias, do)
+    check(got, ref, Tq, grad_mult=3, grad_add=2e-3 if bias_dtype == "fp32" else 0.0, name=f"masked tiles {block}")
+    # keys that no query of their (batch, head) sees get exactly zero gradients
+    dead = mask.all(dim=2)  # (B, H, Tk)
+    dk, dv = got[3].cpu().permute(0, 2, 1, 3), got[4].cpu().permute(0, 2, 1, 3)
+    assert torch.all(dk[dead] == 0) and torch.all(dv[dead] == 0)
+
+
 def test_flash_attn_fully_masked_row_gives_zero():
     g = gen(7)
     q, k, v = (randn(g, 1, 70, 2, 32, dtype=torch.float16) for _ in range(3))
