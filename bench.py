@@ -318,7 +318,8 @@ def attention_case(torch, name, B, T, H, D, dtype, bias_kind, iters=20, with_cpu
     o, dq, dk, dv = (torch.empty_like(q) for _ in range(4))
     tqr = lib.rgd_attn_seqlen_q_rounded(T)
     lse = torch.empty(B, H, tqr, dtype=torch.float32, device="cuda")
-    ws = torch.empty(lib.rgd_attn_bwd_workspace(B, H, T, T, D), dtype=torch.uint8, device="cuda")
+    mode = {"auto": 0, "two_kernel": 1, "one_pass": 2}[os.environ.get("RGD_ATTN_BWD", "auto")]
+    ws = torch.empty(lib.rgd_attn_bwd_workspace(B, H, T, T, D, mode), dtype=torch.uint8, device="cuda")
     fws = torch.empty(max(lib.rgd_attn_fwd_workspace(B, H, T, T, D), 16), dtype=torch.uint8, device="cuda")
     code = _hip.dtype_code(dtype)
     if bias is None:
@@ -336,7 +337,7 @@ def attention_case(torch, name, B, T, H, D, dtype, bias_kind, iters=20, with_cpu
 
     def bwd():
         assert lib.rgd_attn_bwd(B, H, T, T, D, t["do"], t["q"], t["k"], t["v"], t["o"], lse.data_ptr(), bdesc, bk, bd,
-                                t["dq"], t["dk"], t["dv"], code, 0, scale, ws.data_ptr(), ws.numel(), st) == 0, \
+                                t["dq"], t["dk"], t["dv"], code, 0, scale, mode, ws.data_ptr(), ws.numel(), st) == 0, \
             lib.rgd_last_error()
 
     # forward and backward alternate as in a training step; the clocks are brought to their steady state first

@@ -231,21 +231,35 @@ int rgd_attn_fwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D,
  * depend on scheduling; a split item sums its keys in a different grouping than an unsplit one. */
 size_t rgd_attn_fwd_workspace(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D);
 
-/* bytes of scratch for rgd_attn_bwd (any contents on entry, 16-byte aligned): delta, fp32 (B,H,Tq_rounded),
- * which is required, then room for the fp32 partial sums of split workgroups (as in rgd_attn_fwd_workspace),
- * which is optional: a workspace that only holds delta is accepted and nothing is split. */
-size_t rgd_attn_bwd_workspace(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D);
+/* Forms of the attention backward.
+ *   RGD_ATTN_BWD_TWO_KERNEL  a dQ kernel (query blocks) and a dK/dV kernel (key blocks): seven matrix products for the
+ *                            five of the mathematics, no atomics, every result reproducible bit for bit.
+ *   RGD_ATTN_BWD_ONE_PASS    one key-block kernel that also produces dQ by fp32 atomic additions into a dq_accum in the
+ *                            workspace (what the reference sketches with tl.atomic_add in its sequence-parallel
+ *                            branch, flash_attn_triton_cached.py:553-565), head dims up to 64.  dK and dV are
+ *                            reproducible bit for bit; dQ differs from run to run in its last bits (the reference's
+ *                            own race test allows that, tests/test_flash_attn.py:368,383).
+ *   RGD_ATTN_BWD_AUTO        the library's choice for the shape (the one-pass form only if the workspace holds
+ *                            dq_accum). */
+enum rgd_attn_bwd_mode { RGD_ATTN_BWD_AUTO = 0, RGD_ATTN_BWD_TWO_KERNEL = 1, RGD_ATTN_BWD_ONE_PASS = 2 };
+
+/* bytes of scratch for rgd_attn_bwd in the given mode (any contents on entry, 16-byte aligned): delta, fp32
+ * (B,H,Tq_rounded), which is required; for the one-pass form dq_accum, fp32 (B,H,Tq_rounded,D padded to 32 or 64),
+ * required by RGD_ATTN_BWD_ONE_PASS; then room for the fp32 partial sums of split workgroups (as in
+ * rgd_attn_fwd_workspace), which is optional: a smaller workspace is accepted and nothing is split. */
+size_t rgd_attn_bwd_workspace(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, int mode);
 
 /* replaces _flash_attn_backward, flash_attn/flash_attn_triton_cached.py:885-1075
  * (kernels :249-292 and :327-755): delta = rowsum(o*do), P recomputed from lse, dv = P^T do,
  * dS = P*(do v^T - delta)*scale, dk = dS^T q, dq = dS k.  No bias gradient.  dq, dk, dv are written
- * in the tensor dtype from fp32 accumulators, each exactly once, in a fixed order. */
+ * in the tensor dtype from fp32 accumulators, each exactly once; in a fixed order except for dq in the one-pass
+ * form (see rgd_attn_bwd_mode). */
 int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D,
                  const rgd_tensor4* dout, const rgd_tensor4* q, const rgd_tensor4* k,
                  const rgd_tensor4* v, const rgd_tensor4* o, const float* lse,
                  const rgd_tensor4* bias, int bias_kind, int bias_dtype,
                  const rgd_tensor4* dq, const rgd_tensor4* dk, const rgd_tensor4* dv,
-                 int dtype, int causal, float softmax_scale,
+                 int dtype, int causal, float softmax_scale, int mode,
                  void* workspace, size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus

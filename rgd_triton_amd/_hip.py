@@ -18,6 +18,7 @@ HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "rgd_hip.h")
 RGD_F32, RGD_F16, RGD_BF16 = 0, 1, 2
 ABI_MAJOR = 2  # rgd_version() // 1000 this binding was written for
 BIAS_NONE, BIAS_VECTOR, BIAS_MATRIX = 0, 1, 2
+ATTN_BWD_AUTO, ATTN_BWD_TWO_KERNEL, ATTN_BWD_ONE_PASS = 0, 1, 2
 
 _DTYPE_CODE = {torch.float32: RGD_F32, torch.float16: RGD_F16, torch.bfloat16: RGD_BF16}
 
@@ -61,9 +62,9 @@ _SIGNATURES = {
     "rgd_attn_seqlen_q_rounded": (_i64, [_i64]),
     "rgd_attn_fwd": (_int, [_i64] * 5 + [_T4] * 4 + [_int, _int, _T4, _vp, _int, _int, _f32, _vp, _sz, _vp]),
     "rgd_attn_fwd_workspace": (_sz, [_i64] * 5),
-    "rgd_attn_bwd_workspace": (_sz, [_i64] * 5),
-    "rgd_attn_bwd": (_int, [_i64] * 5 + [_T4] * 5 + [_vp] + [_T4, _int, _int] + [_T4] * 3 + [_int, _int, _f32, _vp, _sz,
-                                                                                         _vp]),
+    "rgd_attn_bwd_workspace": (_sz, [_i64] * 5 + [_int]),
+    "rgd_attn_bwd": (_int, [_i64] * 5 + [_T4] * 5 + [_vp] + [_T4, _int, _int] + [_T4] * 3 + [_int, _int, _f32, _int, _vp,
+                                                                                         _sz, _vp]),
 }
 
 _lib = None

@@ -11,6 +11,13 @@ template <typename T> int dispatch_fwd(const AttnFwdParams& p, unsigned grid, hi
 template <typename T> int dispatch_fwd_merge(const AttnFwdParams& p, unsigned items, hipStream_t s);
 template <typename T> int dispatch_bwd_merge(const AttnBwdParams& p, unsigned items, int nt, hipStream_t s);
 template <typename T, bool DQ> int dispatch_bwd(const AttnBwdParams& p, unsigned grid, hipStream_t s);
+template <typename T> int dispatch_bwd_fused(const AttnBwdParams& p, unsigned grid, hipStream_t s);
+template <typename T> int dispatch_bwd_fused_aux(const AttnBwdParams& p, int which, hipStream_t s);
+
+// 1: RGD_ATTN_BWD_AUTO takes the one-pass form where it exists
+#ifndef RGD_ATTN_BWD_AUTO_ONE_PASS
+#define RGD_ATTN_BWD_AUTO_ONE_PASS 0
+#endif
 
 namespace {
 
@@ -37,6 +44,16 @@ int bwd_blocks_per_cu(int dpad) { return dpad <= 64 ? 2 : 1; }           // dK/d
 int dq_blocks_per_cu(int dpad) { return (dpad <= 64 || dpad == 128) ? 2 : 1; }  // dQ kernel (32-key tiles at 128)
 size_t bwd_part_bytes(int dpad, int tensors) { return (size_t)tensors * BWD_BM * dpad * sizeof(float); }
 size_t bwd_delta_bytes(int64_t B, int64_t H, int64_t Tq) { return (size_t)(B * H * rgd_attn_seqlen_q_rounded(Tq)) * sizeof(float); }
+// one-pass form: fp32 dq_accum (B, H, Tq_rounded, DPAD) behind delta
+size_t bwd_accum_bytes(int64_t B, int64_t H, int64_t Tq, int dpad) { return bwd_delta_bytes(B, H, Tq) * (size_t)dpad; }
+// The form a call runs in.  AUTO takes the one-pass form where it exists (head dims up to 64) and the workspace has
+// room for dq_accum; its dQ then depends on the arrival order of atomic additions (last-bit differences from run to
+// run), dK and dV do not.  TWO_KERNEL is reproducible bit for bit.
+bool bwd_one_pass(int mode, int64_t D, size_t workspace_bytes, size_t need) {
+    if (mode == RGD_ATTN_BWD_TWO_KERNEL || D > 64) return false;
+    if (mode == RGD_ATTN_BWD_ONE_PASS) return true;
+    return RGD_ATTN_BWD_AUTO_ONE_PASS && workspace_bytes >= need;
+}
 
 // measured: what a second and third resident workgroup add to a compute unit, and the duration of one inner
 // step (64 keys or 64 query rows) of a workgroup that has its compute unit to itself
@@ -145,18 +162,23 @@ int rgd_attn_fwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
     return RGD_OK;
 }
 
-size_t rgd_attn_bwd_workspace(int64_t B, int64_t H, int64_t Tq, int64_t, int64_t D) {
-    // delta, then room for two rounds of dK/dV parts (the dQ parts reuse it; the launches are ordered)
+size_t rgd_attn_bwd_workspace(int64_t B, int64_t H, int64_t Tq, int64_t, int64_t D, int mode) {
+    // delta, dq_accum where the one-pass form may run, then room for two rounds of dK/dV parts (the dQ parts of the
+    // two-kernel form reuse it; the launches are ordered)
     const int dpad = attn_dpad(D < 1 ? 1 : D);
-    return bwd_delta_bytes(B, H, Tq) + (size_t)2 * rgd_num_cus() * bwd_blocks_per_cu(dpad) * bwd_part_bytes(dpad, 2);
+    const bool accum = mode != RGD_ATTN_BWD_TWO_KERNEL && D <= 64 && (mode == RGD_ATTN_BWD_ONE_PASS || RGD_ATTN_BWD_AUTO_ONE_PASS);
+    return bwd_delta_bytes(B, H, Tq) + (accum ? bwd_accum_bytes(B, H, Tq, dpad) : 0) +
+           (size_t)2 * rgd_num_cus() * bwd_blocks_per_cu(dpad) * bwd_part_bytes(dpad, 2);
 }
 
 int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const rgd_tensor4* dout, const rgd_tensor4* q,
                  const rgd_tensor4* k, const rgd_tensor4* v, const rgd_tensor4* o, const float* lse,
                  const rgd_tensor4* bias, int bias_kind, int bias_dtype, const rgd_tensor4* dq, const rgd_tensor4* dk,
-                 const rgd_tensor4* dv, int dtype, int causal, float softmax_scale, void* workspace,
+                 const rgd_tensor4* dv, int dtype, int causal, float softmax_scale, int mode, void* workspace,
                  size_t workspace_bytes, void* stream) {
     const char* name = "rgd_attn_bwd";
+    RGD_REQUIRE(mode == RGD_ATTN_BWD_AUTO || mode == RGD_ATTN_BWD_TWO_KERNEL || mode == RGD_ATTN_BWD_ONE_PASS,
+                RGD_ERR_INVALID, "%s: bad mode %d", name, mode);
     int rc = check_common(name, B, H, Tq, Tk, D, dtype, bias_kind, bias_dtype, bias);
     if (rc != RGD_OK) return rc;
     if (B * H == 0 || (Tq == 0 && Tk == 0)) return RGD_OK;
@@ -173,10 +195,17 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
     RGD_REQUIRE(workspace_bytes >= delta_bytes && (workspace || Tq == 0), RGD_ERR_WORKSPACE, "%s: workspace too small",
                 name);
     const int dpad = attn_dpad(D);
+    RGD_REQUIRE(mode != RGD_ATTN_BWD_ONE_PASS || D <= 64, RGD_ERR_UNSUPPORTED,
+                "%s: the one-pass form covers head dims up to 64 (got %lld)", name, (long long)D);
+    const size_t accum_bytes = bwd_accum_bytes(B, H, Tq, dpad);
+    const bool one_pass = bwd_one_pass(mode, D, workspace_bytes, delta_bytes + accum_bytes);
+    RGD_REQUIRE(!one_pass || (workspace_bytes >= delta_bytes + accum_bytes && rgd_aligned16(workspace)), RGD_ERR_WORKSPACE,
+                "%s: the one-pass form needs %zu bytes of 16-byte aligned workspace", name, delta_bytes + accum_bytes);
+    const size_t fixed_bytes = delta_bytes + (one_pass ? accum_bytes : 0);
     const bool may_split = workspace && rgd_aligned16(workspace) && !causal;
-    float* part_base = reinterpret_cast<float*>(static_cast<char*>(workspace) + delta_bytes);
-    const size_t part_room = workspace_bytes - delta_bytes;
-    const int per_cu = bwd_blocks_per_cu(dpad);
+    float* part_base = reinterpret_cast<float*>(static_cast<char*>(workspace) + fixed_bytes);
+    const size_t part_room = workspace_bytes - fixed_bytes;
+    const int per_cu = one_pass ? RGD_FUSED_OCC : bwd_blocks_per_cu(dpad);
 
     AttnBwdParams p;
     memset(&p, 0, sizeof(p));
@@ -211,6 +240,36 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
                      (p.bias.sn % per16) == 0;
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (one_pass) {
+        p.dq_accum = reinterpret_cast<float*>(static_cast<char*>(workspace) + delta_bytes);
+        if (Tq > 0) {  // delta, and dq_accum = 0
+            rc = dtype == RGD_F16 ? dispatch_bwd_fused_aux<f16_t>(p, 0, s) : dispatch_bwd_fused_aux<bf16_t>(p, 0, s);
+            if (rc != RGD_OK) return rc;
+        }
+        if (Tk > 0) {  // dK, dV and the dQ contributions of every key block
+            p.nblk = (int)((Tk + BWD_BM - 1) / BWD_BM);
+            const int64_t items = (int64_t)p.nblk * B * H;
+            AttnSplit plan;
+            if (may_split)
+                plan = attn_split_plan(items, rgd_num_cus(), per_cu, (int)((Tq + 63) / 64), bwd_part_bytes(dpad, 2), part_room,
+                                       kBwdSplit);
+            p.split_full = plan.full;
+            p.split_s = plan.s;
+            p.part = part_base;
+            const int64_t grid = plan.blocks(items);
+            RGD_REQUIRE(grid < (1ll << 31), RGD_ERR_UNSUPPORTED, "%s: grid too large", name);
+            rc = dtype == RGD_F16 ? dispatch_bwd_fused<f16_t>(p, (unsigned)grid, s) : dispatch_bwd_fused<bf16_t>(p, (unsigned)grid, s);
+            if (rc != RGD_OK) return rc;
+            if (plan.s > 1) {
+                const unsigned n = (unsigned)plan.items_split(items);
+                rc = dtype == RGD_F16 ? dispatch_bwd_merge<f16_t>(p, n, 2, s) : dispatch_bwd_merge<bf16_t>(p, n, 2, s);
+                if (rc != RGD_OK) return rc;
+            }
+        }
+        if (Tq > 0)  // dq = scale * dq_accum
+            return dtype == RGD_F16 ? dispatch_bwd_fused_aux<f16_t>(p, 1, s) : dispatch_bwd_fused_aux<bf16_t>(p, 1, s);
+        return RGD_OK;
+    }
     if (Tq > 0) {  // dQ and delta
         p.nblk = (int)((Tq + BWD_BM - 1) / BWD_BM);
         const int64_t items = (int64_t)p.nblk * B * H;

@@ -13,6 +13,19 @@
 //       dV^T += dO^T . P            A = dO^T via transposing reads    B = P  (registers)
 //       dK^T += Q^T . dS            A = Q^T  via transposing reads    B = dS (registers)
 //
+//   attn_bwd_dkv_kernel<..., FUSED = true>   the same kernel also produces dQ (one pass, five products instead of
+//                         seven): every wavefront leaves its dS block in LDS, and after the step's barrier the
+//                         wavefronts share out  dQ (32 queries x d) += dS (32 x 128 keys) . K (128 x d),
+//                         A = dS via transposing reads, B = K^T held in registers, and add the result to an fp32
+//                         dq_accum with atomics.  delta comes from attn_bwd_prep_kernel (which also clears dq_accum),
+//                         dQ is rounded and scaled by attn_bwd_dq_convert_kernel.  dK and dV are as deterministic as
+//                         in the two-kernel form; dQ depends on the order in which the key blocks' atomics arrive.
+//                         Measured on MI355X, (4,4096,16,64) bf16: 1.79 ms against 0.93 ms for the two kernels.  The
+//                         atomics are 2.1 GB of fp32 additions (T^2*d*4/128 bytes per batch and head) and the L2 takes
+//                         about 3.2 TB/s of them: 0.66 ms that the rest of the kernel does not hide (timing-only builds:
+//                         0.72 ms without any dQ work, 0.83 with the dS stores, 1.13 with the dQ product, 1.79 with the
+//                         atomics).  It is therefore selectable, not the default.
+//
 // In both kernels the row/column that owns the output (query row for dQ, key for dK/dV) sits in one
 // lane column (lane % 32), so P and dS go from accumulator registers straight into the next matrix
 // product, and all LDS tiles are stored row-major exactly as they arrive from HBM.  The softmax scale
@@ -38,6 +51,7 @@ struct AttnBwdParams {
     // partial sums in `part`, (parts, 128, DPAD) for dQ and (parts, 2, 128, DPAD) for dK, dV
     int split_full, split_s;
     float* part;
+    float* dq_accum;  // one-pass form: fp32 (B, H, Tq_rounded, DPAD), cleared by attn_bwd_prep_kernel
 };
 
 // block id -> (logical item, part, number of parts, part id)
@@ -408,13 +422,31 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
 // Query rows per loop iteration of the dK/dV kernel = 32 * dkv_nsub: each wavefront works on dkv_nsub
 // independent 32-row sub-tiles between two barriers, which gives the scheduler matrix work of one sub-tile
 // to put beside the exponentials of the other.  A bias costs the registers that would take.
-constexpr int dkv_nsub(int dpad, int bias) { return (bias == BIAS_OFF || dpad > 64) ? RGD_DKV_NSUB : 1; }
-template <int DPAD, int NSUB> struct DkvSmem {
+#ifndef RGD_FUSED_NSUB_BIAS
+#define RGD_FUSED_NSUB_BIAS 2
+#endif
+#ifndef RGD_FUSED_OCC
+#define RGD_FUSED_OCC 1  // wavefronts per SIMD of the one-pass kernel
+#endif
+
+constexpr int dkv_nsub(int dpad, int bias, bool fused = false) {
+    return fused ? (bias == BIAS_OFF ? 2 : RGD_FUSED_NSUB_BIAS) : ((bias == BIAS_OFF || dpad > 64) ? RGD_DKV_NSUB : 1);
+}
+constexpr int dkv_occupancy(int dpad, int bias, bool fused) {
+    return fused ? RGD_FUSED_OCC : (dpad <= 64 ? (bias == BIAS_OFF ? RGD_DKV_OCC : 2) : 1);
+}
+template <int DPAD, int NSUB, bool FUSED = false> struct DkvSmem {
     static constexpr int BQ = 32 * NSUB;  // query rows per tile
     static constexpr int TILE = BQ * BwdTile<DPAD>::S;
     // per buffer: Q tile, dO tile, then BQ floats of -lse*log2e and BQ floats of -delta
     static constexpr int BUF_BYTES = 2 * TILE * 2 + 2 * BQ * 4;
-    static constexpr size_t BYTES = 2 * BUF_BYTES;
+    // one-pass form: dS sub-tiles, [128 keys][32 queries + 8] elements each, NSUB per step, two steps deep
+    static constexpr int DS_STRIDE = 40;
+    static constexpr int DS_TILE = BWD_BM * DS_STRIDE;
+    static constexpr int DS_BYTES = FUSED ? 2 * NSUB * DS_TILE * 2 : 0;
+    static constexpr size_t BYTES = 2 * BUF_BYTES + DS_BYTES;
+    // the K tile of the workgroup ([128][S] elements) passes through the Q/dO buffers once, before the first step
+    static_assert(!FUSED || 2 * BUF_BYTES >= BWD_BM * BwdTile<DPAD>::S * 2, "K tile must fit the staging buffers");
 };
 
 // 16 bias values of one key column (16 consecutive rows of the bias matrix) in the "key per lane" layout.
@@ -470,13 +502,19 @@ template <typename TB> struct BiasColumn {
     __device__ __forceinline__ Bits bits(int v) const { return __builtin_bit_cast(Bits, raw[v]); }
 };
 
-template <typename T, int DPAD, int BIAS>
-__global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_DKV_OCC : 2) : 1) void attn_bwd_dkv_kernel(const AttnBwdParams p) {
+template <typename T, int DPAD, int BIAS, bool FUSED = false>
+__global__ __launch_bounds__(BWD_THREADS, dkv_occupancy(DPAD, BIAS, FUSED)) void attn_bwd_dkv_kernel(const AttnBwdParams p) {
     constexpr bool HAS_BIAS = BIAS != BIAS_OFF;
     typedef typename BiasElem<T, BIAS>::type TB;
     typedef Mfma<T> MM;
-    constexpr int NSUB = dkv_nsub(DPAD, BIAS);
-    typedef DkvSmem<DPAD, NSUB> SM;
+    constexpr int NSUB = dkv_nsub(DPAD, BIAS, FUSED);
+    typedef DkvSmem<DPAD, NSUB, FUSED> SM;
+    static_assert(!FUSED || DPAD <= 64, "the one-pass form keeps K^T in registers: head dims up to 64");
+    constexpr int DS_ST = SM::DS_STRIDE;
+    constexpr int DS_TILE = SM::DS_TILE;
+    // dQ work of one step: NSUB query sub-tiles x NDB_ blocks of 32 channels, one item per wavefront
+    constexpr int DQ_ITEMS = FUSED ? NSUB * (DPAD / 32) : 0;
+    static_assert(DQ_ITEMS <= 4, "one dQ item per wavefront");
     constexpr int BQ = SM::BQ;
     constexpr int ST = BwdTile<DPAD>::S;
     constexpr int TILE = SM::TILE;
@@ -521,6 +559,52 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_D
             dk_acc[d][v] = 0.f;
             dv_acc[d][v] = 0.f;
         }
+
+    // ---- one-pass form: K^T of the workgroup's 128 keys as the B operand of the dQ product, dS tiles in LDS ----
+    T* const ds_base = reinterpret_cast<T*>(smem_raw + 2 * BUFB);
+    const int dq_u = wave / NDB, dq_db = wave % NDB;  // this wavefront's dQ item: query sub-tile, block of 32 channels
+    typename MM::V8 ktreg[FUSED ? BWD_BM / 16 : 1];
+    float* dq_dst = nullptr;  // &dq_accum[b, h, 16 * g, this lane's channel]
+    if constexpr (FUSED) {
+        T* kt = reinterpret_cast<T*>(smem_raw);
+        const T* krows = static_cast<const T*>(p.k.ptr) + b * p.k.sb + h * p.k.sh;
+        for (int id = tid; id < BWD_BM * CPR; id += BWD_THREADS) {
+            const int row = id / CPR, dc = id - row * CPR;
+            const int kr = kblk * BWD_BM + row;
+            const u32x4 raw = load8<T>(krows + (int64_t)min(kr, p.Tk - 1) * p.k.sn, dc * 8, p.D, kr < p.Tk, vec);
+            *reinterpret_cast<u32x4*>(kt + row * ST + dc * 8) = raw;
+        }
+        // both parities of the dS tiles start from zero: the first step's dQ phase works on the tile "before" it
+        for (int id = tid; id < SM::DS_BYTES / 16; id += BWD_THREADS)
+            reinterpret_cast<u32x4*>(ds_base)[id] = u32x4{0u, 0u, 0u, 0u};
+        __syncthreads();
+        if (DQ_ITEMS == 4 || wave < DQ_ITEMS) {
+#pragma unroll
+            for (int kk = 0; kk < BWD_BM / 16; ++kk) ktreg[kk] = load_a_transposed<T>(kt, ST, 16 * kk + 8 * g, 32 * dq_db, lane);
+        }
+        __syncthreads();  // the buffers are about to receive the first Q / dO tile
+        dq_dst = p.dq_accum + ((int64_t)bh * p.Tq_rounded + dq_u * 32 + 16 * g) * DPAD + 32 * dq_db + mfma_row_perm(li);
+    }
+    // dQ of the query tile `jprev` (whose dS every wavefront finished before the last barrier):
+    //   dQ (32 x 32 block of this wavefront) = dS (32 queries x 128 keys) . K (128 x 32 channels), added to dq_accum.
+    // Accumulator value v of lane (li, g) is query 16g + v, channel 32 * dq_db + perm(li): for every v the 32 lanes of a
+    // half write 32 consecutive floats.  jprev = -1 (before the first tile) adds the zeros the tiles start from.
+    auto dq_phase = [&](const int jprev) __attribute__((always_inline)) {
+        if constexpr (FUSED) {
+            if (DQ_ITEMS == 4 || wave < DQ_ITEMS) {
+                const T* ds = ds_base + ((jprev & 1) * NSUB + dq_u) * DS_TILE;
+                f32x16 acc;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+#pragma unroll
+                for (int kk = 0; kk < BWD_BM / 16; ++kk)
+                    acc = MM::run(load_a_transposed<T>(ds, DS_ST, 16 * kk + 8 * g, 0, lane), ktreg[kk], acc);
+                float* dst = dq_dst + (int64_t)(max(jprev, 0) * BQ) * DPAD;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) unsafeAtomicAdd(dst + v * DPAD, acc[v]);
+            }
+        }
+    };
 
     // this workgroup's share of the query tiles (all of them unless the item is split)
     const int ntiles_all = (p.Tq + BQ - 1) / BQ;
@@ -647,6 +731,7 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_D
             issue_loads(j + 1, FAST);
             if constexpr (HAS_BIAS) bias_load(b_fill, j + 1, FAST);
         }
+        dq_phase(j - 1);  // one-pass form: dQ of the previous tile, beside this tile's first products
         const T* qs = reinterpret_cast<const T*>(smem_raw + buf * BUFB);
         const T* dos = qs + TILE;
         const float* st = reinterpret_cast<const float*>(smem_raw + buf * BUFB + 2 * TILE * 2);
@@ -754,6 +839,12 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_D
                 pk[v / 2] = pack2<T>(p0, p1);
                 dsk[v / 2] = pack2<T>(p0 * dp[u][v], p1 * dp[u][v + 1]);
             }
+            if constexpr (FUSED) {
+                // dS of this lane's key for queries 16g .. 16g+15 of sub-tile u: one row piece of the [key][query] tile
+                T* dsw = ds_base + ((j & 1) * NSUB + u) * DS_TILE + (wave * 32 + li) * DS_ST + 16 * g;
+                *reinterpret_cast<u32x4*>(dsw) = u32x4{dsk[0], dsk[1], dsk[2], dsk[3]};
+                *reinterpret_cast<u32x4*>(dsw + 8) = u32x4{dsk[4], dsk[5], dsk[6], dsk[7]};
+            }
             // dV^T += dO^T . P ;  dK^T += Q^T . dS
             if constexpr (READ_AHEAD) {
                 u32x4 dta[2], qta[2];  // transposed dO and Q operands, one (jj, d) step ahead
@@ -829,6 +920,9 @@ __global__ __launch_bounds__(BWD_THREADS, DPAD <= 64 ? (BIAS == BIAS_OFF ? RGD_D
         }
         for (; j < ntiles; ++j) tile_step(j, IntC<0>{}, IntC<0>{}, IntC<2>{});
     }
+    if constexpr (FUSED) {
+        if (tile_begin < ntiles) dq_phase(ntiles - 1);  // the last tile's dS is complete: the loop ended on a barrier
+    }
 
     if (item.nparts > 1) {  // part of a split item: leave the unscaled fp32 sums, dK then dV
         float* row = p.part + (((int64_t)item.part_id * 2) * BWD_BM + wave * 32 + li) * DPAD;
@@ -880,5 +974,64 @@ template <typename T, int DPAD> __global__ __launch_bounds__(256) void attn_bwd_
 #pragma unroll
         for (int e = 0; e < 4; ++e)
             if (col + e < p.D) op[col + e] = static_cast<T>(acc[e] * mul);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// one-pass form: before and after the main kernel
+// ------------------------------------------------------------------------------------------------
+// delta[b, h, q] = rowsum(O * dO) for q < Tq (0 for the padding rows up to Tq_rounded) and dq_accum = 0.
+// A row of DPAD channels is handled by DPAD/8 consecutive lanes (16-byte pieces); grid = rows / (256 / (DPAD/8)).
+template <typename T, int DPAD> __global__ __launch_bounds__(256) void attn_bwd_prep_kernel(const AttnBwdParams p) {
+    constexpr int CPR = DPAD / 8;
+    static_assert((CPR & (CPR - 1)) == 0, "lane groups are powers of two");
+    const int64_t row = (int64_t)blockIdx.x * (256 / CPR) + threadIdx.x / CPR;  // over (b, h, Tq_rounded)
+    const int c = threadIdx.x % CPR;
+    if (row >= (int64_t)p.B * p.H * p.Tq_rounded) return;  // whole lane groups leave together
+    const int bh = (int)(row / p.Tq_rounded), q = (int)(row - (int64_t)bh * p.Tq_rounded);
+    const int b = bh / p.H, h = bh - b * p.H;
+    const bool valid = q < p.Tq;
+    const int ql = valid ? q : 0;
+    const T* op = static_cast<const T*>(p.o.ptr) + b * p.o.sb + h * p.o.sh + (int64_t)ql * p.o.sn;
+    const T* dop = static_cast<const T*>(p.dout.ptr) + b * p.dout.sb + h * p.dout.sh + (int64_t)ql * p.dout.sn;
+    const typename Mfma<T>::V8 ov = as_v8<T>(load8<T>(op, c * 8, p.D, valid, p.vec != 0));
+    const typename Mfma<T>::V8 dv = as_v8<T>(load8<T>(dop, c * 8, p.D, valid, p.vec != 0));
+    float sum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sum += static_cast<float>(ov[e]) * static_cast<float>(dv[e]);
+    sum = group_reduce<CPR>(sum);
+    if (c == 0) p.delta[row] = sum;
+    f32x4* acc = reinterpret_cast<f32x4*>(p.dq_accum + row * DPAD + c * 8);
+    acc[0] = f32x4{0.f, 0.f, 0.f, 0.f};
+    acc[1] = f32x4{0.f, 0.f, 0.f, 0.f};
+}
+
+// dq[b, q, h, :] = scale * dq_accum[b, h, q, :], rounded once to the tensor type; one thread per 8 channels
+template <typename T, int DPAD> __global__ __launch_bounds__(256) void attn_bwd_dq_convert_kernel(const AttnBwdParams p) {
+    constexpr int CPR = DPAD / 8;
+    const int64_t row = (int64_t)blockIdx.x * (256 / CPR) + threadIdx.x / CPR;  // over (b, h, Tq)
+    const int c = threadIdx.x % CPR;
+    if (row >= (int64_t)p.B * p.H * p.Tq) return;
+    const int bh = (int)(row / p.Tq), q = (int)(row - (int64_t)bh * p.Tq);
+    const int b = bh / p.H, h = bh - b * p.H;
+    const float* src = p.dq_accum + ((int64_t)bh * p.Tq_rounded + q) * DPAD + c * 8;
+    const f32x4 lo = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(src));
+    const f32x4 hi = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(src) + 1);
+    T* dq = static_cast<T*>(const_cast<void*>(p.dq.ptr)) + b * p.dq.sb + h * p.dq.sh + (int64_t)q * p.dq.sn;
+    const int col = c * 8;
+    if (p.vec) {
+        if (col < p.D) {
+            Pack16 o;
+            o.w[0] = pack2<T>(lo[0] * p.scale, lo[1] * p.scale);
+            o.w[1] = pack2<T>(lo[2] * p.scale, lo[3] * p.scale);
+            o.w[2] = pack2<T>(hi[0] * p.scale, hi[1] * p.scale);
+            o.w[3] = pack2<T>(hi[2] * p.scale, hi[3] * p.scale);
+            *reinterpret_cast<u32x4*>(dq + col) = o.v;
+        }
+    } else {
+        const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            if (col + e < p.D) dq[col + e] = static_cast<T>(v[e] * p.scale);
     }
 }

@@ -6,3 +6,5 @@ template int dispatch_bwd<f16_t, true>(const AttnBwdParams&, unsigned, hipStream
 template int dispatch_bwd<f16_t, false>(const AttnBwdParams&, unsigned, hipStream_t);
 template int dispatch_bwd_merge<f16_t>(const AttnBwdParams&, unsigned, int, hipStream_t);
 template int attn_configure_all<f16_t>();
+template int dispatch_bwd_fused<f16_t>(const AttnBwdParams&, unsigned, hipStream_t);
+template int dispatch_bwd_fused_aux<f16_t>(const AttnBwdParams&, int, hipStream_t);

@@ -43,6 +43,41 @@ template <typename T, int DPAD, int BIAS, bool DQ> int launch_bwd(const AttnBwdP
     return rgd_launch_status("rgd_attn_bwd", rgd_launch(kern, dim3(grid), dim3(BWD_THREADS), lds, s, p));
 }
 
+// ---- one-pass backward (head dims up to 64): prep -> fused key-block kernel -> dQ convert ----
+template <typename T, int DPAD, int BIAS> int launch_bwd_fused(const AttnBwdParams& p, unsigned grid, hipStream_t s) {
+    constexpr size_t lds = DkvSmem<DPAD, dkv_nsub(DPAD, BIAS, true), true>::BYTES;
+    return rgd_launch_status("rgd_attn_bwd (one pass)",
+                             rgd_launch(attn_bwd_dkv_kernel<T, DPAD, BIAS, true>, dim3(grid), dim3(BWD_THREADS), lds, s, p));
+}
+template <typename T> int dispatch_bwd_fused(const AttnBwdParams& p, unsigned grid, hipStream_t s) {
+    const int bias = p.bias_kind == RGD_BIAS_NONE ? BIAS_OFF : (p.bias_dtype == RGD_F32 ? BIAS_F32 : BIAS_SAME);
+#define FUSED_CASE(DP)                                                                 \
+    if (p.D <= DP)                                                                     \
+        return bias == BIAS_OFF    ? launch_bwd_fused<T, DP, BIAS_OFF>(p, grid, s)     \
+               : bias == BIAS_SAME ? launch_bwd_fused<T, DP, BIAS_SAME>(p, grid, s)    \
+                                   : launch_bwd_fused<T, DP, BIAS_F32>(p, grid, s);
+    FUSED_CASE(32)
+    FUSED_CASE(64)
+#undef FUSED_CASE
+    rgd_set_error("rgd_attn_bwd: the one-pass form covers head dims up to 64");
+    return RGD_ERR_UNSUPPORTED;
+}
+// which = 0: delta and a cleared dq_accum before the main kernel; 1: dq from dq_accum after it
+template <typename T> int dispatch_bwd_fused_aux(const AttnBwdParams& p, int which, hipStream_t s) {
+    const int dpad = p.D <= 32 ? 32 : 64;
+    const int rows_per_block = 256 / (dpad / 8);
+    const int64_t rows = (int64_t)p.B * p.H * (which == 0 ? p.Tq_rounded : p.Tq);
+    const dim3 grid((unsigned)((rows + rows_per_block - 1) / rows_per_block));
+    hipError_t e;
+    if (which == 0)
+        e = dpad == 32 ? rgd_launch(attn_bwd_prep_kernel<T, 32>, grid, dim3(256), 0, s, p)
+                       : rgd_launch(attn_bwd_prep_kernel<T, 64>, grid, dim3(256), 0, s, p);
+    else
+        e = dpad == 32 ? rgd_launch(attn_bwd_dq_convert_kernel<T, 32>, grid, dim3(256), 0, s, p)
+                       : rgd_launch(attn_bwd_dq_convert_kernel<T, 64>, grid, dim3(256), 0, s, p);
+    return rgd_launch_status(which == 0 ? "rgd_attn_bwd (prep)" : "rgd_attn_bwd (dq convert)", e);
+}
+
 template <typename T, bool DQ> int dispatch_bwd(const AttnBwdParams& p, unsigned grid, hipStream_t s) {
     const int bias = p.bias_kind == RGD_BIAS_NONE ? BIAS_OFF : (p.bias_dtype == RGD_F32 ? BIAS_F32 : BIAS_SAME);
 #define BWD_CASE(DP)                                                                     \
@@ -75,6 +110,14 @@ template <typename T> int dispatch_bwd_merge(const AttnBwdParams& p, unsigned it
 // launch.  Called once per process from the library's set-up, for every instantiation of this element type, so no
 // entry point touches function attributes afterwards (an entry point may run under stream capture, where such a
 // call is not allowed).
+template <typename T, int DPAD, int BIAS> const void* fused_kernel_ptr() {
+    if constexpr (DPAD <= 64) return reinterpret_cast<const void*>(attn_bwd_dkv_kernel<T, DPAD, BIAS, true>);
+    else return nullptr;
+}
+template <int DPAD, int BIAS> constexpr size_t fused_kernel_lds() {
+    if constexpr (DPAD <= 64) return DkvSmem<DPAD, dkv_nsub(DPAD, BIAS, true), true>::BYTES;
+    else return 0;
+}
 template <typename T, int DPAD, int BIAS> int attn_configure_one() {
     struct K {
         const void* fn;
@@ -84,6 +127,7 @@ template <typename T, int DPAD, int BIAS> int attn_configure_one() {
         {reinterpret_cast<const void*>(attn_fwd_kernel<T, DPAD, BIAS>), AttnFwdSmem<DPAD>::BYTES},
         {reinterpret_cast<const void*>(attn_bwd_dq_kernel<T, DPAD, BIAS>), DqSmem<DPAD>::BYTES},
         {reinterpret_cast<const void*>(attn_bwd_dkv_kernel<T, DPAD, BIAS>), DkvSmem<DPAD, dkv_nsub(DPAD, BIAS)>::BYTES},
+        {fused_kernel_ptr<T, DPAD, BIAS>(), fused_kernel_lds<DPAD, BIAS>()},
     };
     for (const K& k : ks) {
         if (k.lds <= 48 * 1024) continue;

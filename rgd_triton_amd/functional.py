@@ -20,6 +20,7 @@ Differences from the reference, all deliberate:
 """
 import ctypes
 import math
+import os
 
 import torch
 
@@ -29,6 +30,7 @@ from ._hip import t3, t4
 __all__ = [
     "flash_attn_func", "triton_rms_func_fn", "triton_fused_rms_func_fn", "triton_fused_ln_func_fn",
     "triton_norm_func_fn", "triton_fused_norm_func_fn", "triton_rope_fn", "triton_fused_ln_rope_fn",
+    "set_attention_backward",
 ]
 
 _FLOATS = (torch.float16, torch.bfloat16, torch.float32)
@@ -514,6 +516,30 @@ def _flash_attn_forward(q, k, v, bias=None, causal=False, softmax_scale=None, ke
     return o, lse, softmax_scale
 
 
+_ATTN_BWD_MODES = {"auto": _hip.ATTN_BWD_AUTO, "two_kernel": _hip.ATTN_BWD_TWO_KERNEL, "one_pass": _hip.ATTN_BWD_ONE_PASS}
+_attn_bwd_mode = os.environ.get("RGD_ATTN_BWD", "auto")
+assert _attn_bwd_mode in _ATTN_BWD_MODES, f"RGD_ATTN_BWD must be one of {sorted(_ATTN_BWD_MODES)}"
+
+
+def set_attention_backward(mode):
+    """Form of the attention backward: "two_kernel" (every gradient reproducible bit for bit), "one_pass" (head dims up
+    to 64: one kernel, dQ accumulated with fp32 atomics, so its last bits differ from run to run; dK and dV do not;
+    wider heads run the two-kernel form) or "auto" (the library's choice).  `torch.use_deterministic_algorithms(True)`
+    overrides it with "two_kernel".  Returns the previous setting."""
+    global _attn_bwd_mode
+    assert mode in _ATTN_BWD_MODES, f"mode must be one of {sorted(_ATTN_BWD_MODES)}"
+    prev, _attn_bwd_mode = _attn_bwd_mode, mode
+    return prev
+
+
+def _bwd_mode(d):
+    if torch.are_deterministic_algorithms_enabled():
+        return _hip.ATTN_BWD_TWO_KERNEL
+    if _attn_bwd_mode == "one_pass" and d > 64:
+        return _hip.ATTN_BWD_TWO_KERNEL
+    return _ATTN_BWD_MODES[_attn_bwd_mode]
+
+
 def _flash_attn_backward(do, q, k, v, o, lse, dq, dk, dv, bias=None, causal=False, softmax_scale=None,
                          kernel_cache=None):
     if do.stride(-1) != 1:
@@ -530,12 +556,13 @@ def _flash_attn_backward(do, q, k, v, o, lse, dq, dk, dv, bias=None, causal=Fals
     _seen(kernel_cache, "bwd_odot", _sig(o, do))
     softmax_scale = softmax_scale or 1.0 / math.sqrt(d)
     bdesc, bkind, bdtype = _bias_args(bias, q, seqlen_q, seqlen_k, batch, nheads)
-    nbytes = lib.rgd_attn_bwd_workspace(batch, nheads, seqlen_q, seqlen_k, d)
+    mode = _bwd_mode(d)
+    nbytes = lib.rgd_attn_bwd_workspace(batch, nheads, seqlen_q, seqlen_k, d, mode)
     ws = _hip.workspace(q.device, nbytes)
     _hip.check(lib.rgd_attn_bwd(batch, nheads, seqlen_q, seqlen_k, d, t4(do, False), t4(q, False), t4(k, False),
                                 t4(v, False), t4(o, False), ctypes.c_void_p(lse.data_ptr()), bdesc, bkind, bdtype,
                                 t4(dq, False), t4(dk, False), t4(dv, False), _hip.dtype_code(q.dtype),
-                                int(bool(causal)), float(softmax_scale), ws.data_ptr(), nbytes,
+                                int(bool(causal)), float(softmax_scale), mode, ws.data_ptr(), nbytes,
                                 _hip.stream_ptr(q.device)), "rgd_attn_bwd")
 
 

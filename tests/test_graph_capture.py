@@ -34,7 +34,7 @@ class _Sequence:
         self.pe = oracle.rotary_table(T + 1, 32, 10000.0, dt).cuda()
         lib = self.lib
         self.rms_ws = torch.empty(max(lib.rgd_rms_bwd_workspace(B, T, 384, 77, 640), 1), dtype=torch.uint8, device="cuda")
-        self.attn_ws = torch.empty(lib.rgd_attn_bwd_workspace(B, H, T, T, D), dtype=torch.uint8, device="cuda")
+        self.attn_ws = torch.empty(lib.rgd_attn_bwd_workspace(B, H, T, T, D, 1), dtype=torch.uint8, device="cuda")
         self.attn_fws = torch.empty(max(lib.rgd_attn_fwd_workspace(B, H, T, T, D), 16), dtype=torch.uint8, device="cuda")
         self.lse = torch.empty(B, H, lib.rgd_attn_seqlen_q_rounded(T), dtype=torch.float32, device="cuda")
 
@@ -71,7 +71,7 @@ class _Sequence:
                                self.attn_fws.numel(), st)
         rc |= lib.rgd_attn_bwd(B, H, T, T, D, t4(i["g1"]), t4(out["qo"]), t4(out["ko"]), t4(i["v"]), t4(out["o"]),
                                self.lse.data_ptr(), bdesc, hip.BIAS_MATRIX, code, t4(out["dq"]), t4(out["dk"]),
-                               t4(out["dv"]), code, 0, scale, self.attn_ws.data_ptr(), self.attn_ws.numel(), st)
+                               t4(out["dv"]), code, 0, scale, 1, self.attn_ws.data_ptr(), self.attn_ws.numel(), st)
         assert rc == 0, lib.rgd_last_error()
 
 
