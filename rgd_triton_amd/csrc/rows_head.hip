@@ -134,7 +134,9 @@ int head_launch(const char* name, int mode, int64_t B, int64_t H, int64_t Tq, in
     const int rows_per_block = 4 * (64 / cfg.G) * head_unroll(mode, cfg.NV);
     p.blocks_q = (uint32_t)(((int64_t)p.h[0].rows + rows_per_block - 1) / rows_per_block);
     const int64_t blocks = p.blocks_q + ((int64_t)p.h[1].rows + rows_per_block - 1) / rows_per_block;
-    const dim3 grid((unsigned)blocks, 1, 1);
+    p.nblocks = (uint32_t)blocks;
+    const int64_t cap = RGD_HEAD_PERSIST > 0 ? (int64_t)rgd_num_cus() * RGD_HEAD_PERSIST : blocks;
+    const dim3 grid((unsigned)std::min(blocks, cap), 1, 1);
     hipStream_t s = static_cast<hipStream_t>(stream);
     int rc;
     if (dtype == RGD_F32)
