@@ -337,7 +337,7 @@ def attention_case(torch, name, B, T, H, D, dtype, bias_kind, iters=20, with_cpu
 
     def bwd():
         assert lib.rgd_attn_bwd(B, H, T, T, D, t["do"], t["q"], t["k"], t["v"], t["o"], lse.data_ptr(), bdesc, bk, bd,
-                                t["dq"], t["dk"], t["dv"], code, 0, scale, mode, ws.data_ptr(), ws.numel(), st) == 0, \
+                                t["dq"], t["dk"], t["dv"], None, code, 0, scale, mode, ws.data_ptr(), ws.numel(), st) == 0, \
             lib.rgd_last_error()
 
     # forward and backward alternate as in a training step; the clocks are brought to their steady state first

@@ -251,7 +251,12 @@ size_t rgd_attn_bwd_workspace(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int6
 
 /* replaces _flash_attn_backward, flash_attn/flash_attn_triton_cached.py:885-1075
  * (kernels :249-292 and :327-755): delta = rowsum(o*do), P recomputed from lse, dv = P^T do,
- * dS = P*(do v^T - delta)*scale, dk = dS^T q, dq = dS k.  No bias gradient.  dq, dk, dv are written
+ * dS = P*(do v^T - delta)*scale, dk = dS^T q, dq = dS k.
+ * dbias (NULL, or ptr NULL: none; the reference has none, flash_attn_triton_cached.py:1107) receives the bias
+ * gradient P*(do v^T - delta) of every (query, key) pair in the bias dtype: a full (B,H,Tq,Tk) tensor by strides,
+ * 16-byte aligned, rows at least Tk rounded up to 64 elements long (the padding is written too), which the caller
+ * sums over the dimensions its bias broadcasts; with causal != 0 the caller clears it first (key tiles past the
+ * diagonal are not visited).  Two-kernel form only.  dq, dk, dv are written
  * in the tensor dtype from fp32 accumulators, each exactly once; in a fixed order except for dq in the one-pass
  * form (see rgd_attn_bwd_mode). */
 int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D,
@@ -259,6 +264,7 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D,
                  const rgd_tensor4* v, const rgd_tensor4* o, const float* lse,
                  const rgd_tensor4* bias, int bias_kind, int bias_dtype,
                  const rgd_tensor4* dq, const rgd_tensor4* dk, const rgd_tensor4* dv,
+                 const rgd_tensor4* dbias,
                  int dtype, int causal, float softmax_scale, int mode,
                  void* workspace, size_t workspace_bytes, void* stream);
 

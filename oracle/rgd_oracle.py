@@ -18,7 +18,8 @@ the closed-form backward functions follow the reference's kernels.  How each one
                                cutoff 0 / channels >= R, autograd transpose for pair-duplicated tables
   ln_rope_fwd / ln_rope_bwd    composition of the two pinned halves + autograd (fp64)
   attention_fwd / attention_bwd  brute-force python loops in fp64 on tiny inputs, torch.softmax /
-                               torch.logsumexp, autograd (fp64), bias-broadcast equivalence
+                               torch.logsumexp, autograd (fp64, including the bias gradient in every broadcast
+                               form), bias-broadcast equivalence
   attention_lowp               in fp64 it equals attention_fwd and the brute-force loops for every bias form,
                                causal or not, and its autograd gradients equal attention_bwd; in bf16 / fp16 its
                                error lies in a measured band around the rounding error of the exact result
@@ -315,12 +316,14 @@ def attention_fwd(q, k, v, bias=None, causal=False, softmax_scale=None, compute_
     return o.to(q.dtype), lse.to(torch.float32)
 
 
-def attention_bwd(do, q, k, v, bias=None, causal=False, softmax_scale=None, compute_dtype=torch.float32):
+def attention_bwd(do, q, k, v, bias=None, causal=False, softmax_scale=None, compute_dtype=torch.float32,
+                  with_dbias=False):
     """Closed-form gradients as the reference kernels compute them
     (flash_attn_triton_cached.py:249-292 and :426-571):
         delta = rowsum(O * dO);  P = exp(S - LSE);  dV = P^T dO;  dP = dO V^T;
         dS = P * (dP - delta) * scale;  dK = dS^T Q;  dQ = dS K
-    Everything in compute_dtype (no intermediate rounding)."""
+    Everything in compute_dtype (no intermediate rounding).  with_dbias adds the gradient of the bias, which the
+    reference does not provide (:1107): dS / scale, summed over the dimensions the bias broadcasts."""
     s, scale = _scores(q, k, bias, causal, softmax_scale, compute_dtype)
     lse = torch.logsumexp(s, dim=-1)
     dead = torch.isinf(lse)
@@ -334,7 +337,13 @@ def attention_bwd(do, q, k, v, bias=None, causal=False, softmax_scale=None, comp
     ds = p * (dp - delta[..., None]) * scale
     dk = torch.einsum("bhts,bthd->bshd", ds, q.to(compute_dtype))
     dq = torch.einsum("bhts,bshd->bthd", ds, k.to(compute_dtype))
-    return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype)
+    if not with_dbias:
+        return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype)
+    db = p * (dp - delta[..., None])
+    dims = [i for i in range(4) if bias.shape[i] == 1 and db.shape[i] != 1]
+    if dims:
+        db = db.sum(dim=dims, keepdim=True)
+    return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype), db.to(bias.dtype)
 
 
 def attention_lowp(q, k, v, bias=None, causal=False):

@@ -63,7 +63,7 @@ _SIGNATURES = {
     "rgd_attn_fwd": (_int, [_i64] * 5 + [_T4] * 4 + [_int, _int, _T4, _vp, _int, _int, _f32, _vp, _sz, _vp]),
     "rgd_attn_fwd_workspace": (_sz, [_i64] * 5),
     "rgd_attn_bwd_workspace": (_sz, [_i64] * 5 + [_int]),
-    "rgd_attn_bwd": (_int, [_i64] * 5 + [_T4] * 5 + [_vp] + [_T4, _int, _int] + [_T4] * 3 + [_int, _int, _f32, _int, _vp,
+    "rgd_attn_bwd": (_int, [_i64] * 5 + [_T4] * 5 + [_vp] + [_T4, _int, _int] + [_T4] * 4 + [_int, _int, _f32, _int, _vp,
                                                                                          _sz, _vp]),
 }
 

@@ -174,8 +174,8 @@ size_t rgd_attn_bwd_workspace(int64_t B, int64_t H, int64_t Tq, int64_t, int64_t
 int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const rgd_tensor4* dout, const rgd_tensor4* q,
                  const rgd_tensor4* k, const rgd_tensor4* v, const rgd_tensor4* o, const float* lse,
                  const rgd_tensor4* bias, int bias_kind, int bias_dtype, const rgd_tensor4* dq, const rgd_tensor4* dk,
-                 const rgd_tensor4* dv, int dtype, int causal, float softmax_scale, int mode, void* workspace,
-                 size_t workspace_bytes, void* stream) {
+                 const rgd_tensor4* dv, const rgd_tensor4* dbias, int dtype, int causal, float softmax_scale, int mode,
+                 void* workspace, size_t workspace_bytes, void* stream) {
     const char* name = "rgd_attn_bwd";
     RGD_REQUIRE(mode == RGD_ATTN_BWD_AUTO || mode == RGD_ATTN_BWD_TWO_KERNEL || mode == RGD_ATTN_BWD_ONE_PASS,
                 RGD_ERR_INVALID, "%s: bad mode %d", name, mode);
@@ -197,8 +197,21 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
     const int dpad = attn_dpad(D);
     RGD_REQUIRE(mode != RGD_ATTN_BWD_ONE_PASS || D <= 64, RGD_ERR_UNSUPPORTED,
                 "%s: the one-pass form covers head dims up to 64 (got %lld)", name, (long long)D);
+    const bool want_dbias = dbias && dbias->ptr;
+    if (want_dbias) {
+        // written by the dQ kernel as 16-key runs of whole 64-key tiles: rows padded and 16-byte aligned
+        const int64_t per16 = bias_dtype == RGD_F32 ? 4 : 8;
+        RGD_REQUIRE(bias_kind != RGD_BIAS_NONE, RGD_ERR_INVALID, "%s: a bias gradient without a bias", name);
+        RGD_REQUIRE(mode != RGD_ATTN_BWD_ONE_PASS, RGD_ERR_UNSUPPORTED,
+                    "%s: the bias gradient comes from the dQ kernel of the two-kernel form", name);
+        RGD_REQUIRE(dbias->stride_n >= (Tk + 63) / 64 * 64 && dbias->stride_n < (int64_t(1) << 31) &&
+                        rgd_aligned16(dbias->ptr) && dbias->stride_b % per16 == 0 && dbias->stride_h % per16 == 0 &&
+                        dbias->stride_n % per16 == 0,
+                    RGD_ERR_INVALID, "%s: dbias needs 16-byte aligned rows of at least %lld elements (Tk rounded up to 64)",
+                    name, (long long)((Tk + 63) / 64 * 64));
+    }
     const size_t accum_bytes = bwd_accum_bytes(B, H, Tq, dpad);
-    const bool one_pass = bwd_one_pass(mode, D, workspace_bytes, delta_bytes + accum_bytes);
+    const bool one_pass = !want_dbias && bwd_one_pass(mode, D, workspace_bytes, delta_bytes + accum_bytes);
     RGD_REQUIRE(!one_pass || (workspace_bytes >= delta_bytes + accum_bytes && rgd_aligned16(workspace)), RGD_ERR_WORKSPACE,
                 "%s: the one-pass form needs %zu bytes of 16-byte aligned workspace", name, delta_bytes + accum_bytes);
     const size_t fixed_bytes = delta_bytes + (one_pass ? accum_bytes : 0);
@@ -217,6 +230,7 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
     p.dq = at(dq);
     p.dk = at(dk);
     p.dv = at(dv);
+    if (want_dbias) p.dbias = at(dbias);
     p.lse = lse;
     p.delta = static_cast<float*>(workspace);
     p.B = (int)B;

@@ -52,6 +52,9 @@ struct AttnBwdParams {
     int split_full, split_s;
     float* part;
     float* dq_accum;  // one-pass form: fp32 (B, H, Tq_rounded, DPAD), cleared by attn_bwd_prep_kernel
+    // bias gradient (optional, dQ kernel): dS = P * (dP - delta) of every (query, key) pair, in the bias dtype, as a
+    // full (B, H, Tq, Tk) tensor whose rows are padded to whole 64-key tiles (the caller sums broadcast dims)
+    AttnTensor dbias;
 };
 
 // block id -> (logical item, part, number of parts, part id)
@@ -261,8 +264,11 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
     const int a_off = mfma_row_perm(li) * ST + g * 8;
     const int tr_off = ((lane & 15) >> 2) * ST + mfma_row_perm(((lane >> 4) & 1) * 16 + (lane & 3) * 4) + g * 16 * ST;
     const TB* bias_row = nullptr;
+    TB* dbias_row = nullptr;  // this lane's row of the bias gradient, when one is wanted
     BiasRuns<TB, NKB> bias_cur, bias_nxt;  // fetched one tile ahead of use
     if constexpr (HAS_BIAS) {
+        if (p.dbias.ptr)
+            dbias_row = static_cast<TB*>(const_cast<void*>(p.dbias.ptr)) + b * p.dbias.sb + h * p.dbias.sh + (int64_t)q_ld * p.dbias.sn;
         bias_row = static_cast<const TB*>(p.bias.ptr) + b * p.bias.sb + h * p.bias.sh + (int64_t)q_ld * p.bias.sn;
         if (t_begin < t_end) bias_cur.load(bias_row, t_begin * BN, g, p.Tk, p.bias_vec && (t_begin + 1) * BN <= p.Tk);
     }
@@ -339,11 +345,32 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
             for (int v = 0; v < 16; v += 2) {
                 const float p0 = __builtin_amdgcn_exp2f(s[kb][v]);
                 const float p1 = __builtin_amdgcn_exp2f(s[kb][v + 1]);
-                if constexpr (DP_INIT)
-                    dsk[kb][v / 2] = pack2<T>(p0 * dp[kb][v], p1 * dp[kb][v + 1]);
-                else
-                    dsk[kb][v / 2] = pack2<T>(p0 * (dp[kb][v] - delta), p1 * (dp[kb][v + 1] - delta));
+                const float ds0 = DP_INIT ? p0 * dp[kb][v] : p0 * (dp[kb][v] - delta);
+                const float ds1 = DP_INIT ? p1 * dp[kb][v + 1] : p1 * (dp[kb][v + 1] - delta);
+                dsk[kb][v / 2] = pack2<T>(ds0, ds1);
+                if constexpr (BIAS == BIAS_F32) {  // the fp32 values are only needed for an fp32 bias gradient
+                    s[kb][v] = ds0;
+                    s[kb][v + 1] = ds1;
+                }
             }
+        if constexpr (HAS_BIAS) {
+            if (dbias_row != nullptr && q_valid) {
+                // bias gradient: this lane's query row, 16 consecutive keys per 32-key half (rows are padded to whole
+                // tiles, so the runs of a ragged last tile stay inside the row)
+#pragma unroll
+                for (int kb = 0; kb < NKB; ++kb) {
+                    TB* dst = dbias_row + key0 + kb * 32 + g * 16;
+                    if constexpr (BIAS == BIAS_F32) {
+#pragma unroll
+                        for (int e = 0; e < 16; e += 4)
+                            *reinterpret_cast<f32x4*>(dst + e) = f32x4{s[kb][e], s[kb][e + 1], s[kb][e + 2], s[kb][e + 3]};
+                    } else {
+                        *reinterpret_cast<u32x4*>(dst) = u32x4{dsk[kb][0], dsk[kb][1], dsk[kb][2], dsk[kb][3]};
+                        *reinterpret_cast<u32x4*>(dst + 8) = u32x4{dsk[kb][4], dsk[kb][5], dsk[kb][6], dsk[kb][7]};
+                    }
+                }
+            }
+        }
         // dQ^T += K^T . dS^T
         const T* kt = ks_base + buf * TILE + tr_off;
 #pragma unroll
@@ -360,7 +387,16 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
                 acc[d] = MM::run(as_v8<T>(a), bop, acc[d]);
             }
         }
-        }  // !masked_tile
+        } else if constexpr (HAS_BIAS) {
+            if (dbias_row != nullptr && q_valid) {  // a block that was left out has dS = 0
+#pragma unroll
+                for (int kb = 0; kb < NKB; ++kb) {
+                    u32x4* dst = reinterpret_cast<u32x4*>(dbias_row + key0 + kb * 32 + g * 16);
+#pragma unroll
+                    for (int i = 0; i < (int)(16 * sizeof(TB) / 16); ++i) dst[i] = u32x4{0u, 0u, 0u, 0u};
+                }
+            }
+        }
         if (F || j + 1 < t_end) {
             store_tiles(buf ^ 1, IntC<(AH == 0 ? 0 : 2 - AH)>{});
             if constexpr (HAS_BIAS) bias_cur = bias_nxt;

@@ -541,7 +541,10 @@ def _bwd_mode(d):
 
 
 def _flash_attn_backward(do, q, k, v, o, lse, dq, dk, dv, bias=None, causal=False, softmax_scale=None,
-                         kernel_cache=None):
+                         kernel_cache=None, bias_grad=False):
+    """Returns None, or with bias_grad the gradient of `bias` in its own shape and dtype (beyond the reference, which
+    refuses it, flash_attn_triton_cached.py:1107): the dQ kernel leaves dS of every (query, key) pair in a full
+    (B, H, Tq, Tk) buffer and the dimensions the bias broadcasts are summed here in fp32."""
     if do.stride(-1) != 1:
         do = do.contiguous()
     batch, seqlen_q, nheads, d = q.shape
@@ -557,13 +560,27 @@ def _flash_attn_backward(do, q, k, v, o, lse, dq, dk, dv, bias=None, causal=Fals
     softmax_scale = softmax_scale or 1.0 / math.sqrt(d)
     bdesc, bkind, bdtype = _bias_args(bias, q, seqlen_q, seqlen_k, batch, nheads)
     mode = _bwd_mode(d)
+    dfull, ddesc = None, None
+    if bias_grad:
+        mode = _hip.ATTN_BWD_TWO_KERNEL  # the dQ kernel writes the bias gradient
+        tk_pad = (seqlen_k + 63) // 64 * 64  # rows of whole 64-key tiles
+        alloc = torch.zeros if causal else torch.empty  # key tiles past the causal diagonal are not visited
+        dfull = alloc((batch, nheads, seqlen_q, tk_pad), dtype=bias.dtype, device=q.device)
+        ddesc = _hip.Tensor4(dfull.data_ptr(), dfull.stride(0), dfull.stride(1), dfull.stride(2))
     nbytes = lib.rgd_attn_bwd_workspace(batch, nheads, seqlen_q, seqlen_k, d, mode)
     ws = _hip.workspace(q.device, nbytes)
     _hip.check(lib.rgd_attn_bwd(batch, nheads, seqlen_q, seqlen_k, d, t4(do, False), t4(q, False), t4(k, False),
                                 t4(v, False), t4(o, False), ctypes.c_void_p(lse.data_ptr()), bdesc, bkind, bdtype,
-                                t4(dq, False), t4(dk, False), t4(dv, False), _hip.dtype_code(q.dtype),
+                                t4(dq, False), t4(dk, False), t4(dv, False), ddesc, _hip.dtype_code(q.dtype),
                                 int(bool(causal)), float(softmax_scale), mode, ws.data_ptr(), nbytes,
                                 _hip.stream_ptr(q.device)), "rgd_attn_bwd")
+    if not bias_grad:
+        return None
+    dfull = dfull[..., :seqlen_k]
+    dims = [i for i in range(4) if bias.shape[i] == 1 and dfull.shape[i] != 1]
+    if dims:
+        return dfull.sum(dim=dims, keepdim=True, dtype=torch.float32).to(bias.dtype)
+    return dfull.contiguous()
 
 
 class FlashAttnFunc(torch.autograd.Function):
@@ -587,11 +604,13 @@ class FlashAttnFunc(torch.autograd.Function):
     def backward(ctx, do, dlse):
         _no_capture("FlashAttnFunc.backward")
         q, k, v, o, lse, bias = ctx.saved_tensors
-        assert not ctx.needs_input_grad[3], "FlashAttention does not support bias gradient yet"
+        # the reference stops here with "FlashAttention does not support bias gradient yet"
+        # (flash_attn_triton_cached.py:1107); this implementation provides it
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-        _flash_attn_backward(do, q, k, v, o, lse, dq, dk, dv, bias=bias, causal=ctx.causal,
-                             softmax_scale=ctx.softmax_scale, kernel_cache=ctx.kernel_cache)
-        return dq, dk, dv, None, None, None, None
+        dbias = _flash_attn_backward(do, q, k, v, o, lse, dq, dk, dv, bias=bias, causal=ctx.causal,
+                                     softmax_scale=ctx.softmax_scale, kernel_cache=ctx.kernel_cache,
+                                     bias_grad=bias is not None and ctx.needs_input_grad[3])
+        return dq, dk, dv, dbias, None, None, None
 
 
 def flash_attn_func(q, k, v, bias=None, causal=False, softmax_scale=None, return_lse=False, kernel_cache=None):

@@ -449,10 +449,45 @@ def test_flash_attn_module_errors_and_cache():
         flash_attn_func(big, big, big)
     with pytest.raises(RuntimeError, match="Last 2 dimensions of bias"):
         flash_attn_func(q, q, q, torch.zeros(1, 1, 3, 64, device="cuda", dtype=torch.float16))
-    bias = torch.zeros(1, 1, 64, 64, device="cuda", dtype=torch.float16, requires_grad=True)
-    out = flash_attn_func(q, q, q, bias)
-    with pytest.raises(AssertionError, match="does not support bias gradient"):
-        out.sum().backward()
+
+
+@pytest.mark.parametrize("dtype", HALF)
+@pytest.mark.parametrize("bias_dtype", ["same", "fp32"])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("bias_type", ["static", "batch", "head", "cube", "vector"])
+@pytest.mark.parametrize("d,Tq,Tk", [(64, 113, 203), (32, 200, 130), (128, 256, 320), (59, 97, 64), (64, 1, 239)])
+def test_flash_attn_bias_gradient(d, Tq, Tk, bias_type, causal, bias_dtype, dtype):
+    """The gradient of the bias (the reference refuses it, flash_attn_triton_cached.py:1107): dS = P * (dP - delta) of
+    every pair, summed over the dimensions the bias broadcasts, against the oracle's closed form (pinned by fp64
+    autograd).  The other gradients are unchanged by asking for it."""
+    from rgd_triton_amd import flash_attn_func
+
+    g = gen(14)
+    B, H = 2, 3
+    q, k, v = randn(g, B, Tq, H, d, dtype=dtype), randn(g, B, Tk, H, d, dtype=dtype), randn(g, B, Tk, H, d, dtype=dtype)
+    bt = torch.float32 if bias_dtype == "fp32" else dtype
+    bias = make_bias(g, bias_type, B, H, Tq, Tk, torch.float32)
+    bias[..., Tk // 3] = float("-inf")  # a masked key: zero gradient there
+    bias = bias.to(bt)
+    do = randn(g, B, Tq, H, d, dtype=dtype)
+    qg, kg, vg = to_gpu(q, k, v, requires_grad=True)
+    bg = bias.cuda().requires_grad_(True)
+    o = flash_attn_func(qg, kg, vg, bg, causal)
+    dq, dk, dv, db = torch.autograd.grad(o, (qg, kg, vg, bg), do.cuda())
+    dq2, dk2, dv2 = torch.autograd.grad(flash_attn_func(qg, kg, vg, bg.detach(), causal), (qg, kg, vg), do.cuda())
+    assert torch.equal(dq, dq2) and torch.equal(dk, dk2) and torch.equal(dv, dv2)
+    ref = oracle.attention_bwd(do, q, k, v, bias, causal, None, with_dbias=True)[3]
+    assert db.shape == bias.shape and db.dtype == bias.dtype and not torch.isnan(db).any()
+    assert torch.all(db[..., Tk // 3] == 0)
+    # Error model: an element is a sum of `terms` values dS = P * (dP - delta), each rounded to the operand type (a few
+    # half-ulps of the largest |dS|), and delta = rowsum(O * dO) is formed from the O the forward stored, i.e. rounded
+    # to the tensor type as in the reference's kernel (flash_attn_triton_cached.py:249-292), while the oracle keeps O
+    # in fp32: that moves dP - delta by about half an ulp of |O| |dO| ~ sqrt(d).
+    terms = max(1, (B * H * Tq * Tk) // ref.numel())
+    scale = oracle.attention_bwd(do, q, k, v, bias.expand(B, H, Tq, Tk).contiguous(), causal, None,
+                                 with_dbias=True)[3].float().abs().max().item()
+    allowed = half_ulp(dtype) * (4 * scale + d ** 0.5) * terms ** 0.5
+    assert maxdiff(db, ref) <= allowed, f"dbias error {maxdiff(db, ref)} (allowed {allowed}, scale {scale}, {terms} terms)"
 
 
 @pytest.mark.parametrize("dtype", HALF)
@@ -497,7 +532,7 @@ def test_flash_attn_split_workgroups(B, H, T, d, with_bias, mode, dtype):
                               fws.data_ptr() if fws_bytes else None, fws_bytes, st)
         assert rc == 0, lib.rgd_last_error()
         rc = lib.rgd_attn_bwd(B, H, T, T, d, t["do"], t["q"], t["k"], t["v"], t["o"], lse.data_ptr(), bdesc, bk, bd, t["dq"],
-                              t["dk"], t["dv"], code, 0, scale, mode, bws.data_ptr(), bws_bytes, st)
+                              t["dk"], t["dv"], None, code, 0, scale, mode, bws.data_ptr(), bws_bytes, st)
         assert rc == 0, lib.rgd_last_error()
         torch.cuda.synchronize()
         return o, lse, dq, dk, dv

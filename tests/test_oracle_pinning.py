@@ -244,6 +244,22 @@ def test_attention_backward_against_autograd(causal):
     torch.testing.assert_close(lse.double(), torch.logsumexp(s.detach(), -1), rtol=1e-6, atol=1e-6)
 
 
+@pytest.mark.parametrize("bias_shape", [(1, 1, 7, 9), (2, 1, 7, 9), (1, 3, 7, 9), (2, 3, 7, 9), (2, 3, 1, 9), (1, 1, 1, 9)])
+@pytest.mark.parametrize("causal", [False, True])
+def test_attention_bias_gradient_against_autograd(bias_shape, causal):
+    g = gen(23)
+    q, k, v, do = r64(g, 2, 7, 3, 8), r64(g, 2, 9, 3, 8), r64(g, 2, 9, 3, 8), r64(g, 2, 7, 3, 8)
+    bias = r64(g, *bias_shape).requires_grad_(True)
+    s = torch.einsum("bthd,bshd->bhts", q, k) * 0.3 + bias
+    if causal:
+        s = s.masked_fill(torch.arange(7)[:, None] < torch.arange(9)[None, :], -math.inf)
+    o = torch.einsum("bhts,bshd->bthd", torch.softmax(s, -1), v)
+    (db_ad,) = torch.autograd.grad(o, (bias,), do)
+    got = oracle.attention_bwd(do, q, k, v, bias.detach(), causal, 0.3, F64, with_dbias=True)
+    assert got[3].shape == bias.shape
+    torch.testing.assert_close(got[3], db_ad, rtol=1e-9, atol=1e-12)
+
+
 def test_attention_defaults_and_dead_rows():
     g = gen(8)
     q, k, v = r64(g, 1, 3, 1, 16), r64(g, 1, 4, 1, 16), r64(g, 1, 4, 1, 16)
