@@ -124,9 +124,13 @@ template <int DPAD> struct DqSmem {
     static constexpr size_t BYTES = 2 * 2 * TILE * 2;  // K and V, double buffered
 };
 
-template <typename T, int DPAD, int BIAS>
+// DBIAS: also write the bias gradient (a variant of its own: the kernels for head dims above 64 have no register to
+// spare, and a pointer that is only tested at run time already costs them spills in the main loop: config-4-sized
+// backward 0.31 -> 0.57 ms when it was a run-time option)
+template <typename T, int DPAD, int BIAS, bool DBIAS = false>
 __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32) ? 2 : 1) void attn_bwd_dq_kernel(const AttnBwdParams p) {
     constexpr bool HAS_BIAS = BIAS != BIAS_OFF;
+    static_assert(!DBIAS || HAS_BIAS, "a bias gradient needs a bias");
     typedef typename BiasElem<T, BIAS>::type TB;
     typedef Mfma<T> MM;
     constexpr int BN = DqSmem<DPAD>::BN;
@@ -264,10 +268,10 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
     const int a_off = mfma_row_perm(li) * ST + g * 8;
     const int tr_off = ((lane & 15) >> 2) * ST + mfma_row_perm(((lane >> 4) & 1) * 16 + (lane & 3) * 4) + g * 16 * ST;
     const TB* bias_row = nullptr;
-    TB* dbias_row = nullptr;  // this lane's row of the bias gradient, when one is wanted
+    TB* dbias_row = nullptr;  // this lane's row of the bias gradient (DBIAS)
     BiasRuns<TB, NKB> bias_cur, bias_nxt;  // fetched one tile ahead of use
     if constexpr (HAS_BIAS) {
-        if (p.dbias.ptr)
+        if constexpr (DBIAS)
             dbias_row = static_cast<TB*>(const_cast<void*>(p.dbias.ptr)) + b * p.dbias.sb + h * p.dbias.sh + (int64_t)q_ld * p.dbias.sn;
         bias_row = static_cast<const TB*>(p.bias.ptr) + b * p.bias.sb + h * p.bias.sh + (int64_t)q_ld * p.bias.sn;
         if (t_begin < t_end) bias_cur.load(bias_row, t_begin * BN, g, p.Tk, p.bias_vec && (t_begin + 1) * BN <= p.Tk);
@@ -348,13 +352,13 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
                 const float ds0 = DP_INIT ? p0 * dp[kb][v] : p0 * (dp[kb][v] - delta);
                 const float ds1 = DP_INIT ? p1 * dp[kb][v + 1] : p1 * (dp[kb][v + 1] - delta);
                 dsk[kb][v / 2] = pack2<T>(ds0, ds1);
-                if constexpr (BIAS == BIAS_F32) {  // the fp32 values are only needed for an fp32 bias gradient
+                if constexpr (DBIAS && BIAS == BIAS_F32) {  // the fp32 values are only needed for an fp32 bias gradient
                     s[kb][v] = ds0;
                     s[kb][v + 1] = ds1;
                 }
             }
-        if constexpr (HAS_BIAS) {
-            if (dbias_row != nullptr && q_valid) {
+        if constexpr (DBIAS) {
+            if (q_valid) {
                 // bias gradient: this lane's query row, 16 consecutive keys per 32-key half (rows are padded to whole
                 // tiles, so the runs of a ragged last tile stay inside the row)
 #pragma unroll
@@ -387,8 +391,8 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
                 acc[d] = MM::run(as_v8<T>(a), bop, acc[d]);
             }
         }
-        } else if constexpr (HAS_BIAS) {
-            if (dbias_row != nullptr && q_valid) {  // a block that was left out has dS = 0
+        } else if constexpr (DBIAS) {
+            if (q_valid) {  // a block that was left out has dS = 0
 #pragma unroll
                 for (int kb = 0; kb < NKB; ++kb) {
                     u32x4* dst = reinterpret_cast<u32x4*>(dbias_row + key0 + kb * 32 + g * 16);

@@ -38,8 +38,13 @@ template <typename T> int dispatch_fwd(const AttnFwdParams& p, unsigned grid, hi
 }
 
 template <typename T, int DPAD, int BIAS, bool DQ> int launch_bwd(const AttnBwdParams& p, unsigned grid, hipStream_t s) {
-    auto kern = DQ ? attn_bwd_dq_kernel<T, DPAD, BIAS> : attn_bwd_dkv_kernel<T, DPAD, BIAS>;
     constexpr size_t lds = DQ ? DqSmem<DPAD>::BYTES : DkvSmem<DPAD, dkv_nsub(DPAD, BIAS)>::BYTES;
+    if constexpr (DQ && BIAS != BIAS_OFF) {
+        if (p.dbias.ptr)  // the variant that also writes the bias gradient
+            return rgd_launch_status("rgd_attn_bwd", rgd_launch(attn_bwd_dq_kernel<T, DPAD, BIAS, true>, dim3(grid),
+                                                                dim3(BWD_THREADS), lds, s, p));
+    }
+    auto kern = DQ ? attn_bwd_dq_kernel<T, DPAD, BIAS> : attn_bwd_dkv_kernel<T, DPAD, BIAS>;
     return rgd_launch_status("rgd_attn_bwd", rgd_launch(kern, dim3(grid), dim3(BWD_THREADS), lds, s, p));
 }
 
@@ -110,6 +115,10 @@ template <typename T> int dispatch_bwd_merge(const AttnBwdParams& p, unsigned it
 // launch.  Called once per process from the library's set-up, for every instantiation of this element type, so no
 // entry point touches function attributes afterwards (an entry point may run under stream capture, where such a
 // call is not allowed).
+template <typename T, int DPAD, int BIAS> const void* dq_dbias_kernel_ptr() {
+    if constexpr (BIAS != BIAS_OFF) return reinterpret_cast<const void*>(attn_bwd_dq_kernel<T, DPAD, BIAS, true>);
+    else return nullptr;
+}
 template <typename T, int DPAD, int BIAS> const void* fused_kernel_ptr() {
     if constexpr (DPAD <= 64) return reinterpret_cast<const void*>(attn_bwd_dkv_kernel<T, DPAD, BIAS, true>);
     else return nullptr;
@@ -126,11 +135,12 @@ template <typename T, int DPAD, int BIAS> int attn_configure_one() {
     const K ks[] = {
         {reinterpret_cast<const void*>(attn_fwd_kernel<T, DPAD, BIAS>), AttnFwdSmem<DPAD>::BYTES},
         {reinterpret_cast<const void*>(attn_bwd_dq_kernel<T, DPAD, BIAS>), DqSmem<DPAD>::BYTES},
+        {dq_dbias_kernel_ptr<T, DPAD, BIAS>(), DqSmem<DPAD>::BYTES},
         {reinterpret_cast<const void*>(attn_bwd_dkv_kernel<T, DPAD, BIAS>), DkvSmem<DPAD, dkv_nsub(DPAD, BIAS)>::BYTES},
         {fused_kernel_ptr<T, DPAD, BIAS>(), fused_kernel_lds<DPAD, BIAS>()},
     };
     for (const K& k : ks) {
-        if (k.lds <= 48 * 1024) continue;
+        if (k.fn == nullptr || k.lds <= 48 * 1024) continue;
         if (hipFuncSetAttribute(k.fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)k.lds) != hipSuccess) {
             (void)hipGetLastError();
             rgd_set_error("rgd_init: cannot reserve %zu bytes of LDS for an attention kernel", k.lds);
