@@ -462,6 +462,9 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
 // Query rows per loop iteration of the dK/dV kernel = 32 * dkv_nsub: each wavefront works on dkv_nsub
 // independent 32-row sub-tiles between two barriers, which gives the scheduler matrix work of one sub-tile
 // to put beside the exponentials of the other.  A bias costs the registers that would take.
+#ifndef RGD_DKV_NSUB_BIAS_WIDE
+#define RGD_DKV_NSUB_BIAS_WIDE 2  // sub-tiles per step with a bias at head dims above 64
+#endif
 #ifndef RGD_FUSED_NSUB_BIAS
 #define RGD_FUSED_NSUB_BIAS 2
 #endif
@@ -470,7 +473,8 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
 #endif
 
 constexpr int dkv_nsub(int dpad, int bias, bool fused = false) {
-    return fused ? (bias == BIAS_OFF ? 2 : RGD_FUSED_NSUB_BIAS) : ((bias == BIAS_OFF || dpad > 64) ? RGD_DKV_NSUB : 1);
+    return fused ? (bias == BIAS_OFF ? 2 : RGD_FUSED_NSUB_BIAS)
+                 : (bias == BIAS_OFF ? RGD_DKV_NSUB : (dpad > 64 ? RGD_DKV_NSUB_BIAS_WIDE : 1));
 }
 constexpr int dkv_occupancy(int dpad, int bias, bool fused) {
     return fused ? RGD_FUSED_OCC : (dpad <= 64 ? (bias == BIAS_OFF ? RGD_DKV_OCC : 2) : 1);
@@ -792,7 +796,9 @@ __global__ __launch_bounds__(BWD_THREADS, dkv_occupancy(DPAD, BIAS, FUSED)) void
         // The operand reads run one step ahead of the matrix instructions that use them (the scheduling barriers keep
         // them there).  Left alone, the compiler issues each read right before its use, and with one wavefront per
         // SIMD (head dims above 64) nothing else covers the LDS round trip.  With two wavefronts it makes no difference.
-        constexpr bool READ_AHEAD = RGD_DKV_READ_AHEAD && DPAD > 64;
+        // (not with a bias: the 32 registers of the look-ahead push that variant into spills, and without them the
+        // config-4-sized backward is 2.5 % shorter)
+        constexpr bool READ_AHEAD = RGD_DKV_READ_AHEAD && DPAD > 64 && !HAS_BIAS;
         if constexpr (READ_AHEAD) {
             u32x4 qa[2][NSUB], da[2][NSUB];
             auto read_step = [&](int c) __attribute__((always_inline)) {
