@@ -93,12 +93,12 @@ def timed_loop(torch, step_fns, steps, warmup):
     # (an event between two launches costs a few microseconds of stream time, which is why this is a
     # separate pass and not the one `value` comes from).  A fourth event recorded straight after the third
     # measures that cost (event to event with nothing between); it is subtracted from both intervals.
-    evs = []
-    for i in range(steps):
-        rec = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+    # (the events are created beforehand: creating them inside the loop costs the host more per step than the GPU
+    # needs for it, and an interval then includes the wait for the host)
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(steps)]
+    for i, rec in enumerate(evs):
         step_fns[(i + steps) % n](rec)
         rec[3].record()
-        evs.append(rec)
     torch.cuda.synchronize()
     gap = statistics.median(e[2].elapsed_time(e[3]) for e in evs)
     fwd = [e[0].elapsed_time(e[1]) - gap for e in evs]
