@@ -340,6 +340,34 @@ def test_flash_attn_race_condition(Tq, Tk, bias_type, d):
     assert_repeats_bit_exact(step, ("o", "lse", "dq", "dk", "dv"))
 
 
+DETERMINISTIC_PAIRS = [(1, 239), (3, 799), (127, 512), (127, 513), (113, 203), (128, 217), (113, 211), (108, 256),
+                       (256, 512), (1023, 1024)]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("bias_type", ["none", "cube"])
+@pytest.mark.parametrize("d", [32, 64])
+@pytest.mark.parametrize("swap_sq_sk", [False, True])
+@pytest.mark.parametrize("Tq,Tk", DETERMINISTIC_PAIRS)
+def test_flash_attn_deterministic(Tq, Tk, swap_sq_sk, d, bias_type, dtype):
+    """The test the reference carries but skips ("Determinism not implemented", tests/test_flash_attn.py:546-609):
+    batch 4, 9 heads, its ten (Tq, Tk) pairs both ways round, 50 repeats of the backward of one forward; dq, dk and
+    dv must have the bits of the first run every time.  The two-kernel backward writes every gradient element once."""
+    from rgd_triton_amd import flash_attn_func
+
+    if swap_sq_sk:
+        Tq, Tk = Tk, Tq
+    g = gen(14)
+    B, H = 4, 9
+    q, k, v = randn(g, B, Tq, H, d, dtype=dtype), randn(g, B, Tk, H, d, dtype=dtype), randn(g, B, Tk, H, d, dtype=dtype)
+    bias = make_bias(g, bias_type, B, H, Tq, Tk, dtype)
+    do = randn(g, B, Tq, H, d, dtype=dtype).to("cuda")
+    qg, kg, vg = to_gpu(q, k, v, requires_grad=True)
+    bg = None if bias is None else bias.to("cuda")
+    out = flash_attn_func(qg, kg, vg, bg, False, None, return_lse=False)
+    assert_repeats_bit_exact(lambda: torch.autograd.grad(out, (qg, kg, vg), do, retain_graph=True), ("dq", "dk", "dv"), iters=50)
+
+
 @pytest.fixture
 def one_pass():
     """the one-pass backward (dQ through fp32 atomics) for the duration of a test"""

@@ -114,3 +114,30 @@ def test_l2_norm_race_condition(T, C, dtype):
         return (y, *torch.autograd.grad(y, (xg,), dy))
 
     assert_repeats_bit_exact(step, ("y", "dx"))
+
+
+FUSED_RACE_PAIRS = [(1, 239), (239, 1), (3, 799), (799, 3), (1024, 128), (97, 97), (128, 128), (200, 200), (256, 256),
+                    (257, 257), (384, 384), (512, 512), (768, 768), (1024, 1024)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("d,dfactor", [(32, -0.75), (97, -0.3), (257, 0.2), (510, 0.6), (1023, 1.0)])
+@pytest.mark.parametrize("Tq,Tk", FUSED_RACE_PAIRS)
+def test_fused_l2_norm_race_condition(Tq, Tk, d, dfactor, dtype):
+    """The race test of tests/test_fused_l2normalize.py:283-354: batch 60, its 14 (Tq, Tk) pairs, 250 repeats of forward
+    + backward; the widths follow its rule (dfactor < 0 narrows the first input, else the second).  One (d, dfactor)
+    pairing per width instead of its full 9 x 5 grid."""
+    from rgd_triton_amd import triton_fused_norm_func_fn
+
+    CQ, CK = (int(-dfactor * d), d) if dfactor < 0 else (d, int(dfactor * d))
+    torch.manual_seed(5)  # inputs made on the GPU: nothing here is compared with the CPU oracle
+    B = 60
+    qg, kg, gq, gk = (torch.randn(B, T, C, device="cuda", dtype=dtype) for T, C in ((Tq, CQ), (Tk, CK), (Tq, CQ), (Tk, CK)))
+    qg.requires_grad_(True)
+    kg.requires_grad_(True)
+
+    def step():
+        y = triton_fused_norm_func_fn(qg, kg)
+        return (*y, *torch.autograd.grad(y, (qg, kg), (gq, gk)))
+
+    assert_repeats_bit_exact(step, ("qo", "ko", "dq", "dk"))
