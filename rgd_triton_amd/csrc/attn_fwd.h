@@ -20,9 +20,14 @@
 // rare after the first tiles.  p = exp2(t) <= 256 is safe for fp16/bf16 operands and fp32 sums, and
 // LSE = (m + log2(l)) * ln2 does not depend on where m sits.
 #pragma once
-// 1: the main loop of the forward without bias (d <= 64) fetches two tiles ahead
+// 1: the main loop of the forward at d <= 64 fetches its K/V tiles two tiles ahead
 #ifndef RGD_FWD_PREFETCH2
 #define RGD_FWD_PREFETCH2 1
+#endif
+// ... also with a bias (the bias itself stays one tile ahead).  The biased kernels run two wavefronts per SIMD either
+// way, so the second staging set costs no occupancy; (2,4352,24,64) with a (B,1,Q,K) bias: forward 0.368 -> 0.357 ms.
+#ifndef RGD_FWD_PREFETCH2_BIAS
+#define RGD_FWD_PREFETCH2_BIAS 1
 #endif
 #ifndef RGD_FWD_LAZY_MAX
 #define RGD_FWD_LAZY_MAX 1
@@ -158,7 +163,7 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
     // rows made of whole 16-byte chunks: straight-line loads, no masking except in the last tile
     const bool fast_tiles = vec && p.D % 8 == 0;
     // two staging register sets when the main loop fetches two tiles ahead (PF2), else one
-    constexpr bool PF2 = RGD_FWD_PREFETCH2 && DPAD <= 64 && !HAS_BIAS;
+    constexpr bool PF2 = RGD_FWD_PREFETCH2 && DPAD <= 64 && (!HAS_BIAS || RGD_FWD_PREFETCH2_BIAS);
     u32x4 kst_[PF2 ? 2 : 1][LOADS], vst_[PF2 ? 2 : 1][LOADS];
     // FAST (compile time): the caller knows the tile is full and the 16-byte path applies, so the loads are
     // straight-line code.  The main loop below runs on FAST steps only: with the element-wise loader of ragged
