@@ -124,6 +124,7 @@ int rgd_attn_fwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
     p.Tq_rounded = (int)rgd_attn_seqlen_q_rounded(Tq);
     p.nqb = (int)((Tq + ATTN_BM - 1) / ATTN_BM);
     p.causal = causal ? 1 : 0;
+    p.group_lg = causal_group_lg(causal != 0, B * H);
     p.vec = (D % 8 == 0) && t4_vec_ok(q) && (Tk == 0 || (t4_vec_ok(k) && t4_vec_ok(v))) && t4_vec_ok(o);
     p.scale_log2 = softmax_scale * kLog2e;
     p.bias_kind = bias_kind;
@@ -240,6 +241,7 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
     p.D = (int)D;
     p.Tq_rounded = (int)rgd_attn_seqlen_q_rounded(Tq);
     p.causal = causal ? 1 : 0;
+    p.group_lg = causal_group_lg(causal != 0, B * H);
     p.vec = (D % 8 == 0);
     for (const rgd_tensor4* t : all) p.vec = p.vec && (t->ptr == nullptr || t4_vec_ok(t));
     p.scale = softmax_scale;

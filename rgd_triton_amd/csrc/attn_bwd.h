@@ -50,6 +50,7 @@ struct AttnBwdParams {
     // hardware blocks >= split_full are part (id % split_s) of item split_full + id / split_s and leave fp32
     // partial sums in `part`, (parts, 128, DPAD) for dQ and (parts, 2, 128, DPAD) for dK, dV
     int split_full, split_s;
+    int group_lg;  // dQ launch: see row_block_of
     float* part;
     float* dq_accum;  // one-pass form: fp32 (B, H, Tq_rounded, DPAD), cleared by attn_bwd_prep_kernel
     // bias gradient (optional, dQ kernel): dS = P * (dP - delta) of every (query, key) pair, in the bias dtype, as a
@@ -74,6 +75,22 @@ __device__ __forceinline__ BwdItem bwd_item(const AttnBwdParams& p) {
         it.nparts = p.split_s;
     }
     return it;
+}
+
+#ifndef RGD_DKV_GROUP
+#define RGD_DKV_GROUP 4
+#endif
+// Item of the dK/dV launch -> (key block, batch*head).  Items run through groups of RGD_DKV_GROUP (batch, head) pairs
+// key block by key block: where the work of a key block falls with its index (causal launches, block-causal biases: the
+// first key blocks see every query row) the launch then starts with the long workgroups of several heads and ends on
+// the short ones, instead of giving a late, long workgroup to the compute unit that finished a short one first.
+__device__ __forceinline__ void dkv_block_of(int item, const AttnBwdParams& p, int& kblk, int& bh) {
+    const int nbh = p.B * p.H;
+    const int per = RGD_DKV_GROUP * p.nblk;
+    const int grp = item / per, local = item - grp * per;
+    const int heads = min(RGD_DKV_GROUP, nbh - grp * RGD_DKV_GROUP);
+    kblk = local / heads;
+    bh = grp * RGD_DKV_GROUP + local - kblk * heads;
 }
 
 // 16 contiguous columns of one row of an fp32 partial tile
@@ -154,8 +171,8 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 31, g = lane >> 5;
     const BwdItem item = bwd_item(p);
     const int bid = item.bid;
-    const int qb = p.causal ? p.nblk - 1 - bid % p.nblk : bid % p.nblk;  // causal: longest row blocks first
-    const int bh = bid / p.nblk;
+    int qb, bh;
+    row_block_of(bid, p.nblk, p.group_lg, p.causal != 0, qb, bh);  // causal: longest row blocks first
     const int b = bh / p.H, h = bh - b * p.H;
     const int q_row = qb * BWD_BM + wave * 32 + li;
     const bool q_valid = q_row < p.Tq;
@@ -574,8 +591,8 @@ __global__ __launch_bounds__(BWD_THREADS, dkv_occupancy(DPAD, BIAS, FUSED)) void
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 31, g = lane >> 5;
     const BwdItem item = bwd_item(p);
     const int bid = item.bid;
-    const int kblk = bid % p.nblk;
-    const int bh = bid / p.nblk;
+    int kblk, bh;
+    dkv_block_of(bid, p, kblk, bh);
     const int b = bh / p.H, h = bh - b * p.H;
     const int key = kblk * BWD_BM + wave * 32 + li;  // this lane's key
     const bool k_valid = key < p.Tk;
@@ -1000,7 +1017,9 @@ template <typename T, int DPAD> __global__ __launch_bounds__(256) void attn_bwd_
     const int row = id / CPR, col = (id - row * CPR) * 4;
     const int which = blockIdx.z;
     const int item = p.split_full + blockIdx.x;
-    const int blk = item % p.nblk, bh = item / p.nblk;
+    int blk, bh;
+    if (nt == 2) dkv_block_of(item, p, blk, bh);
+    else row_block_of(item, p.nblk, p.group_lg, p.causal != 0, blk, bh);
     const int b = bh / p.H, h = bh - b * p.H;
     const int t_row = blk * BWD_BM + row;
     const AttnTensor& out = nt == 1 ? p.dq : (which == 0 ? p.dk : p.dv);

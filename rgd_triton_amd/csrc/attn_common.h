@@ -197,6 +197,24 @@ __device__ __forceinline__ int xcd_remap(int id, int n) {
     return x < rem ? x * (per + 1) + slot : rem * (per + 1) + (x - rem) * per + slot;
 }
 
+#ifndef RGD_CAUSAL_GROUP_LOG2
+#define RGD_CAUSAL_GROUP_LOG2 2
+#endif
+// Forward and dQ kernel: item -> (row block, batch*head).  Causal launches: the last row blocks of a (batch, head) have
+// the most key tiles.  Their items run through groups of 4 (batch, head) pairs row block by row block, last row block
+// first (group_lg = 2, set by the host when batch*head is a multiple of 4), so a launch starts on the long workgroups of
+// several heads and ends on short ones; (8,2048,16,64) causal: forward 115 -> 106 us, backward 294 -> 276 us.
+// Otherwise (group_lg = 0) one (batch, head) after the other.  One code path for both: a second path costs the
+// forward without bias registers it does not have (config-3 forward +4 %).
+__device__ __forceinline__ void row_block_of(int item, int nblk, int group_lg, bool last_first, int& blk, int& bh) {
+    const int per = nblk << group_lg;
+    const int grp = item / per, local = item - grp * per;
+    const int pos = local >> group_lg;
+    blk = last_first ? nblk - 1 - pos : pos;
+    bh = (grp << group_lg) + (local & ((1 << group_lg) - 1));
+}
+inline int causal_group_lg(bool causal, int64_t nbh) { return causal && nbh % (1 << RGD_CAUSAL_GROUP_LOG2) == 0 ? RGD_CAUSAL_GROUP_LOG2 : 0; }
+
 struct AttnTensor {
     const void* ptr;
     int64_t sb, sh, sn;

@@ -51,6 +51,7 @@ struct AttnFwdParams {
     // are whole items; the others are part (id % split_s) of item split_full + id / split_s and leave
     // unnormalised partial results, which attn_fwd_merge_kernel combines.  split_s <= 1: no split.
     int split_full, split_s;
+    int group_lg;  // see row_block_of
     float* part_o;   // (parts, 128, DPAD) fp32 accumulators, relative to the part's reference exponent
     float* part_ml;  // (parts, 128, 2): reference exponent (log2 domain), sum of probabilities
 };
@@ -98,10 +99,8 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
         part = part_id % p.split_s;
         nparts = p.split_s;
     }
-    // causal: the last row blocks of a (batch, head) have the most key tiles; they go first, so that the launch
-    // does not end on its longest workgroups
-    const int qb = p.causal ? p.nqb - 1 - bid % p.nqb : bid % p.nqb;
-    const int bh = bid / p.nqb;
+    int qb, bh;
+    row_block_of(bid, p.nqb, p.group_lg, p.causal != 0, qb, bh);
     const int b = bh / p.H;
     const int h = bh - b * p.H;
 
@@ -565,7 +564,8 @@ template <typename T, int DPAD> __global__ __launch_bounds__(256) void attn_fwd_
     if (id >= ATTN_BM * CPR) return;
     const int row = id / CPR, col = (id - row * CPR) * 4;
     const int item = p.split_full + blockIdx.x;
-    const int qb = item % p.nqb, bh = item / p.nqb;
+    int qb, bh;
+    row_block_of(item, p.nqb, p.group_lg, p.causal != 0, qb, bh);
     const int b = bh / p.H, h = bh - b * p.H;
     const int q_row = qb * ATTN_BM + row;
     const int64_t part0 = (int64_t)blockIdx.x * p.split_s;
