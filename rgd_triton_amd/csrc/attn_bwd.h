@@ -129,6 +129,9 @@ __device__ __forceinline__ void store_row16(T* row, int col, int D, bool vec, co
 // ------------------------------------------------------------------------------------------------
 #ifndef RGD_DQ_BN128
 #define RGD_DQ_BN128 32
+#ifndef RGD_DQ_SKIP_EARLY
+#define RGD_DQ_SKIP_EARLY 1
+#endif
 #endif
 // 1: the main loop of the dQ kernel without bias (d <= 64) fetches two tiles ahead
 #ifndef RGD_DQ_PREFETCH2
@@ -311,8 +314,15 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
         }
         const T* ks = ks_base + buf * TILE + a_off;
         const T* vs = vs_base + buf * TILE + a_off;
+        // A tile whose bias is -inf for every (query, key) pair of this wavefront has P = 0 and dS = 0: the step is left
+        // out.  RGD_DQ_SKIP_EARLY 1: tested before the first two products (the bias was requested a step earlier), 0: after.
+        bool masked_tile = false;
+#if RGD_DQ_SKIP_EARLY
+        if constexpr (attn_skip_masked(DPAD, BIAS)) masked_tile = bias_cur.all_neg_inf(0, NKB);
+#endif
         // the dP accumulators start from -delta, so that product comes out as dP - delta
         f32x16 s[NKB], dp[NKB];
+        if (!masked_tile) {
 #pragma unroll
         for (int kb = 0; kb < NKB; ++kb) {
 #pragma unroll
@@ -331,11 +341,10 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
                 dp[kb] = MM::run(as_v8<T>(va), doreg[c], dp[kb]);
             }
         }
-        // A tile whose bias is -inf for every (query, key) pair of this wavefront has P = 0 and dS = 0: the rest of
-        // the step is left out.  Tested where the bias is first needed, after the first two products have been
-        // issued, so the bias loads keep the time of those products to arrive.
-        bool masked_tile = false;
+        }
+#if !RGD_DQ_SKIP_EARLY
         if constexpr (attn_skip_masked(DPAD, BIAS)) masked_tile = bias_cur.all_neg_inf(0, NKB);
+#endif
         if (!masked_tile) {
         float bias_v[NKB][16];
         if constexpr (HAS_BIAS) bias_cur.decode(bias_v);

@@ -29,6 +29,11 @@
 #ifndef RGD_FWD_PREFETCH2_BIAS
 #define RGD_FWD_PREFETCH2_BIAS 1
 #endif
+// 1: the forward (head dims above 64) looks for an all -inf half tile before its first product, 0: after it.  The bias
+// was requested a step earlier; config 4 forward -2 %, a bias without -inf blocks unchanged.
+#ifndef RGD_FWD_SKIP_EARLY
+#define RGD_FWD_SKIP_EARLY 1
+#endif
 #ifndef RGD_FWD_LAZY_MAX
 #define RGD_FWD_LAZY_MAX 1
 #endif
@@ -392,6 +397,12 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb) {
                 // ---- S^T = K . Q^T ----
+                // a half whose bias is -inf everywhere for this wavefront adds nothing and is left out
+#if RGD_FWD_SKIP_EARLY
+                if constexpr (attn_skip_masked(DPAD, BIAS)) {
+                    if (bias_cur.all_neg_inf(kb, 1)) continue;
+                }
+#endif
                 f32x16 s;
 #pragma unroll
                 for (int v = 0; v < 16; ++v) s[v] = 0.f;
@@ -400,11 +411,11 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
                     const u32x4 a = *reinterpret_cast<const u32x4*>(ks + kb * 32 * ST + c * 16);
                     s = MM::run(as_v8<T>(a), qreg[c], s);
                 }
-                // a half whose bias is -inf everywhere for this wavefront adds nothing: its softmax and second
-                // product are left out (tested where the bias is first needed, see above)
+#if !RGD_FWD_SKIP_EARLY
                 if constexpr (attn_skip_masked(DPAD, BIAS)) {
                     if (bias_cur.all_neg_inf(kb, 1)) continue;
                 }
+#endif
 
                 // ---- t = logit - m_ref (log2 domain) ----
                 const float m_off = m_ref == -INFINITY ? 0.f : m_ref;
