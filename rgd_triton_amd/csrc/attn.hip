@@ -35,6 +35,9 @@ AttnTensor at(const rgd_tensor4* t) {
 
 int attn_dpad(int64_t D) { return D <= 32 ? 32 : D <= 64 ? 64 : D <= 96 ? 96 : 128; }
 // resident workgroups per compute unit of the forward kernel (its launch bounds and LDS use)
+#ifndef RGD_GROUP_SHARED_BIAS
+#define RGD_GROUP_SHARED_BIAS 1
+#endif
 int fwd_blocks_per_cu(int dpad, bool bias) { return (dpad <= 64 && !bias) ? 3 : 2; }
 // bytes one part of a split forward item leaves behind: 128 rows of accumulators, exponent and row sum
 size_t fwd_part_bytes(int dpad) { return (size_t)ATTN_BM * dpad * sizeof(float) + (size_t)ATTN_BM * 2 * sizeof(float); }
@@ -124,7 +127,9 @@ int rgd_attn_fwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
     p.Tq_rounded = (int)rgd_attn_seqlen_q_rounded(Tq);
     p.nqb = (int)((Tq + ATTN_BM - 1) / ATTN_BM);
     p.causal = causal ? 1 : 0;
-    p.group_lg = causal_group_lg(causal != 0, B * H);
+    // (a bias matrix shared by the heads of a batch is also read once for four heads that way)
+    const bool bias_shared = RGD_GROUP_SHARED_BIAS && bias_kind == RGD_BIAS_MATRIX && bias->stride_h == 0 && H % 4 == 0;
+    p.group_lg = causal_group_lg(causal != 0 || bias_shared, B * H);
     p.vec = (D % 8 == 0) && t4_vec_ok(q) && (Tk == 0 || (t4_vec_ok(k) && t4_vec_ok(v))) && t4_vec_ok(o);
     p.scale_log2 = softmax_scale * kLog2e;
     p.bias_kind = bias_kind;
@@ -241,7 +246,9 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
     p.D = (int)D;
     p.Tq_rounded = (int)rgd_attn_seqlen_q_rounded(Tq);
     p.causal = causal ? 1 : 0;
-    p.group_lg = causal_group_lg(causal != 0, B * H);
+    // (a bias matrix shared by the heads of a batch is also read once for four heads that way)
+    const bool bias_shared = RGD_GROUP_SHARED_BIAS && bias_kind == RGD_BIAS_MATRIX && bias->stride_h == 0 && H % 4 == 0;
+    p.group_lg = causal_group_lg(causal != 0 || bias_shared, B * H);
     p.vec = (D % 8 == 0);
     for (const rgd_tensor4* t : all) p.vec = p.vec && (t->ptr == nullptr || t4_vec_ok(t));
     p.scale = softmax_scale;
