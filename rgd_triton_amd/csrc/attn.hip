@@ -150,6 +150,10 @@ int rgd_attn_fwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
                                (int)((Tk + ATTN_BN - 1) / ATTN_BN), fwd_part_bytes(dpad), workspace_bytes, kFwdSplit);
     p.split_full = plan.full;
     p.split_s = plan.s;
+    // Leaving leading / trailing all -inf bias tiles out of a workgroup's loop takes a pass over its bias first.  It pays
+    // when workgroups queue for compute units (the launch is then bound by the sum of their work); in a launch of one
+    // round the time is that of the longest workgroup, which has no such tiles and only pays for the search.
+    p.trim = items > (int64_t)rgd_num_cus() * fwd_blocks_per_cu(dpad, bias_kind != RGD_BIAS_NONE);
     if (plan.s > 1) {
         const size_t parts = (size_t)plan.items_split(items) * plan.s;
         p.part_o = static_cast<float*>(workspace);
@@ -302,6 +306,7 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
                                    bwd_part_bytes(dpad, 1), part_room, kBwdSplit);
         p.split_full = plan.full;
         p.split_s = plan.s;
+        p.trim = items > (int64_t)rgd_num_cus() * dq_blocks_per_cu(dpad);  // see rgd_attn_fwd
         p.part = part_base;
         const int64_t grid = plan.blocks(items);
         RGD_REQUIRE(grid < (1ll << 31), RGD_ERR_UNSUPPORTED, "%s: grid too large", name);
@@ -322,6 +327,7 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
                                    kBwdSplit);
         p.split_full = plan.full;
         p.split_s = plan.s;
+        p.trim = items > (int64_t)rgd_num_cus() * per_cu;
         p.part = part_base;
         const int64_t grid = plan.blocks(items);
         RGD_REQUIRE(grid < (1ll << 31), RGD_ERR_UNSUPPORTED, "%s: grid too large", name);

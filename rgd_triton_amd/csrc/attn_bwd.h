@@ -51,6 +51,7 @@ struct AttnBwdParams {
     // partial sums in `part`, (parts, 128, DPAD) for dQ and (parts, 2, 128, DPAD) for dK, dV
     int split_full, split_s;
     int group_lg;  // dQ launch: see row_block_of
+    int trim;      // this launch looks for leading (dK/dV) or trailing (dQ) all -inf bias tiles first
     float* part;
     float* dq_accum;  // one-pass form: fp32 (B, H, Tq_rounded, DPAD), cleared by attn_bwd_prep_kernel
     // bias gradient (optional, dQ kernel): dS = P * (dP - delta) of every (query, key) pair, in the bias dtype, as a
@@ -77,6 +78,9 @@ __device__ __forceinline__ BwdItem bwd_item(const AttnBwdParams& p) {
     return it;
 }
 
+#ifndef RGD_DKV_SKIP_PREFIX
+#define RGD_DKV_SKIP_PREFIX 1
+#endif
 #ifndef RGD_DKV_GROUP
 #define RGD_DKV_GROUP 4
 #endif
@@ -129,6 +133,9 @@ __device__ __forceinline__ void store_row16(T* row, int col, int D, bool vec, co
 // ------------------------------------------------------------------------------------------------
 #ifndef RGD_DQ_BN128
 #define RGD_DQ_BN128 32
+#ifndef RGD_DQ_TRIM
+#define RGD_DQ_TRIM 1
+#endif
 #ifndef RGD_DQ_SKIP_EARLY
 #define RGD_DQ_SKIP_EARLY 1
 #endif
@@ -217,7 +224,16 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
     if (p.causal) ntiles = min(ntiles, (min(p.Tq, (qb + 1) * BWD_BM) + BN - 1) / BN);
     // this workgroup's share of the key tiles (all of them unless the item is split)
     const int t_begin = (int)((int64_t)ntiles * item.part / item.nparts);
-    const int t_end = (int)((int64_t)ntiles * (item.part + 1) / item.nparts);
+    int t_end = (int)((int64_t)ntiles * (item.part + 1) / item.nparts);
+    // trailing key tiles with nothing but -inf in the bias are left out (not when the bias gradient is written: it has
+    // zeros to put there)
+    if constexpr (attn_skip_masked(DPAD, BIAS) && !DBIAS && RGD_DQ_TRIM) {
+        if (p.trim && p.bias_vec && !p.causal && p.Tk % BN == 0 && t_begin < t_end) {
+            const int row0 = qb * BWD_BM + __builtin_amdgcn_readfirstlane(wave) * 32;
+            const TB* rows = static_cast<const TB*>(p.bias.ptr) + b * p.bias.sb + h * p.bias.sh + (int64_t)min(row0, p.Tq - 1) * p.bias.sn;
+            t_end = bias_trim_end<TB, BN>(rows, p.bias.sn, min(32, p.Tq - row0), t_begin, t_end, lane, tid, reinterpret_cast<int*>(smem_raw));
+        }
+    }
 
     const T* kbase = static_cast<const T*>(p.k.ptr) + b * p.k.sb + h * p.k.sh;
     const T* vbase = static_cast<const T*>(p.v.ptr) + b * p.v.sb + h * p.v.sh;
@@ -679,8 +695,58 @@ __global__ __launch_bounds__(BWD_THREADS, dkv_occupancy(DPAD, BIAS, FUSED)) void
     // this workgroup's share of the query tiles (all of them unless the item is split)
     const int ntiles_all = (p.Tq + BQ - 1) / BQ;
     const int tile_first = p.causal ? min(ntiles_all, (kblk * BWD_BM) / BQ) : 0;
-    const int tile_begin = tile_first + (int)((int64_t)(ntiles_all - tile_first) * item.part / item.nparts);
+    int tile_begin = tile_first + (int)((int64_t)(ntiles_all - tile_first) * item.part / item.nparts);
     const int ntiles = tile_first + (int)((int64_t)(ntiles_all - tile_first) * (item.part + 1) / item.nparts);
+
+    // Leading query tiles whose bias is -inf for every (query, key) pair of the workgroup give P = 0 and add nothing to dK
+    // and dV (a block-causal bias: all queries before the key block).  They are found here, before anything else is
+    // loaded, and left out of the loop altogether: every wavefront reads its [BQ rows][32 keys] bias blocks four steps at
+    // a time, 16 bytes per lane, until it meets a value above -inf; the workgroup starts at the earliest such step.
+    // (Inside the loop such a step still costs its tile loads, its first two products and a barrier.)
+    if constexpr (attn_skip_masked(DPAD, BIAS) && !FUSED && RGD_DKV_SKIP_PREFIX) {
+        if (p.trim && p.bias_vec && !p.causal && (kblk + 1) * BWD_BM <= p.Tk && tile_begin < ntiles) {
+            constexpr int EPC = 16 / (int)sizeof(TB);  // bias elements per 16 bytes
+            constexpr int CPW = 32 / EPC;              // 16-byte chunks of the wavefront's 32 keys in a row
+            constexpr int RPL = 64 / CPW;              // rows per load instruction
+            constexpr int LPS = BQ / RPL;              // load instructions per step
+            constexpr int BATCH = 4;
+            constexpr uint32_t PAT = NegInfBits<TB>::value;
+            const TB* col = static_cast<const TB*>(p.bias.ptr) + b * p.bias.sb + h * p.bias.sh + kblk * BWD_BM + wave * 32 +
+                            (lane % CPW) * EPC;
+            const int rsub = lane / CPW;
+            int live = ntiles;  // this wavefront's first step with a value above -inf
+            for (int t0 = tile_begin; t0 < ntiles && live == ntiles; t0 += BATCH) {
+                u32x4 v[BATCH][LPS];
+#pragma unroll
+                for (int bi = 0; bi < BATCH; ++bi)
+#pragma unroll
+                    for (int i = 0; i < LPS; ++i) {
+                        const int row = min(min(t0 + bi, ntiles - 1) * BQ + i * RPL + rsub, p.Tq - 1);
+                        v[bi][i] = *reinterpret_cast<const u32x4*>(col + (int64_t)row * p.bias.sn);
+                    }
+#pragma unroll
+                for (int bi = BATCH - 1; bi >= 0; --bi) {
+                    uint32_t all_and = PAT, all_or = PAT;
+#pragma unroll
+                    for (int i = 0; i < LPS; ++i)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            all_and &= v[bi][i][e];
+                            all_or |= v[bi][i][e];
+                        }
+                    const bool some = __builtin_amdgcn_ballot_w64(all_and != PAT || all_or != PAT) != 0;
+                    if (some && t0 + bi < ntiles) live = t0 + bi;
+                }
+            }
+            int* first_live = reinterpret_cast<int*>(smem_raw);
+            if (tid == 0) *first_live = ntiles;
+            __syncthreads();
+            if (lane == 0) atomicMin(first_live, live);
+            __syncthreads();
+            tile_begin = *first_live;
+            __syncthreads();  // the tile buffers are written next
+        }
+    }
 
     // chunks past the end of a row (head dim below the padded one): as in the dQ kernel
     const bool padded = p.D != DPAD;

@@ -161,6 +161,60 @@ template <typename TB, int NKB = 2> struct BiasRuns {
     }
 };
 
+// Forward and dQ kernel: trailing key tiles whose bias is -inf for every (query, key) pair of the workgroup give P = 0
+// and add nothing (a block-causal bias: all keys after the query block).  Returns the end of [t_begin, t_end) without
+// them, found before anything else is loaded: every wavefront reads its [32 rows][BN keys] bias blocks backwards from
+// the last tile, four tiles at a time and 16 bytes per lane (whole rows by neighbouring lanes), until it meets a value
+// above -inf; the workgroup keeps the tiles up to the latest such tile.  (Inside the loop such a tile still costs its
+// K/V loads and a barrier.)  wave_rows: &bias[b, h, first row of the wavefront, 0]; rows: how many of its 32 rows exist;
+// slot: an int in LDS that nothing else uses until the next barrier after the call.  All tiles must be full tiles.
+template <typename TB, int BN>
+__device__ __forceinline__ int bias_trim_end(const TB* __restrict__ wave_rows, int64_t sn, int rows, int t_begin, int t_end, int lane,
+                                             int tid, int* slot) {
+    constexpr int EPC = 16 / (int)sizeof(TB);
+    constexpr int CPR = BN / EPC;   // 16-byte chunks per row of a tile
+    constexpr int RPL = 64 / CPR;   // rows per load instruction
+    constexpr int LPT = 32 / RPL;   // load instructions per tile
+    constexpr int BATCH = 4;
+    constexpr uint32_t PAT = NegInfBits<TB>::value;
+    int last = t_begin;  // end of this wavefront's live tiles
+    if (rows > 0) {
+        const TB* col = wave_rows + (lane % CPR) * EPC;
+        const int rsub = lane / CPR;
+        for (int t1 = t_end; t1 > t_begin && last == t_begin; t1 -= BATCH) {
+            u32x4 v[BATCH][LPT];
+#pragma unroll
+            for (int bi = 0; bi < BATCH; ++bi)
+#pragma unroll
+                for (int i = 0; i < LPT; ++i) {
+                    const int tile = max(t1 - 1 - bi, t_begin);
+                    const int row = min(i * RPL + rsub, rows - 1);
+                    v[bi][i] = *reinterpret_cast<const u32x4*>(col + (int64_t)row * sn + tile * BN);
+                }
+#pragma unroll
+            for (int bi = BATCH - 1; bi >= 0; --bi) {  // ends on the latest tile of the batch
+                uint32_t all_and = PAT, all_or = PAT;
+#pragma unroll
+                for (int i = 0; i < LPT; ++i)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        all_and &= v[bi][i][e];
+                        all_or |= v[bi][i][e];
+                    }
+                const bool some = __builtin_amdgcn_ballot_w64(all_and != PAT || all_or != PAT) != 0;
+                if (some && t1 - 1 - bi >= t_begin) last = t1 - bi;
+            }
+        }
+    }
+    if (tid == 0) *slot = t_begin;
+    __syncthreads();
+    if (lane == 0) atomicMax(slot, last);
+    __syncthreads();
+    const int end = *slot;
+    __syncthreads();  // the slot's memory is free again
+    return end;
+}
+
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 
 // 4 elements for this lane out of a transposing read; `p` is this lane's own 8-byte source piece

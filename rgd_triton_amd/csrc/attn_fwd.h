@@ -34,6 +34,9 @@
 #ifndef RGD_FWD_SKIP_EARLY
 #define RGD_FWD_SKIP_EARLY 1
 #endif
+#ifndef RGD_FWD_TRIM
+#define RGD_FWD_TRIM 1
+#endif
 #ifndef RGD_FWD_LAZY_MAX
 #define RGD_FWD_LAZY_MAX 1
 #endif
@@ -57,6 +60,7 @@ struct AttnFwdParams {
     // unnormalised partial results, which attn_fwd_merge_kernel combines.  split_s <= 1: no split.
     int split_full, split_s;
     int group_lg;  // see row_block_of
+    int trim;      // look for trailing all -inf bias tiles first (see bias_trim_end)
     float* part_o;   // (parts, 128, DPAD) fp32 accumulators, relative to the part's reference exponent
     float* part_ml;  // (parts, 128, 2): reference exponent (log2 domain), sum of probabilities
 };
@@ -131,7 +135,16 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
     int ntiles = (p.Tk + ATTN_BN - 1) / ATTN_BN;
     if (p.causal) ntiles = min(ntiles, (min(p.Tq, (qb + 1) * ATTN_BM) + ATTN_BN - 1) / ATTN_BN);
     // this workgroup's share of the key tiles (all of them unless the item is split)
-    const int t_begin = (int)((int64_t)ntiles * part / nparts), t_end = (int)((int64_t)ntiles * (part + 1) / nparts);
+    const int t_begin = (int)((int64_t)ntiles * part / nparts);
+    int t_end = (int)((int64_t)ntiles * (part + 1) / nparts);
+    if constexpr (attn_skip_masked(DPAD, BIAS) && RGD_FWD_TRIM) {
+        if (p.trim && p.bias_vec && !p.causal && p.Tk % ATTN_BN == 0 && t_begin < t_end) {
+            const int row0 = qb * ATTN_BM + __builtin_amdgcn_readfirstlane(wave) * 32;
+            const TB* rows = static_cast<const TB*>(p.bias.ptr) + b * p.bias.sb + h * p.bias.sh + (int64_t)min(row0, p.Tq - 1) * p.bias.sn;
+            t_end = bias_trim_end<TB, ATTN_BN>(rows, p.bias.sn, min(32, p.Tq - row0), t_begin, t_end, lane, tid,
+                                               reinterpret_cast<int*>(smem_raw));
+        }
+    }
 
     // global -> register staging of the next tile.  Thread t moves the 16-byte chunks t, t+256, ... of the
     // tile; its offsets inside a tile are fixed, the tile base is wavefront-uniform.

@@ -299,6 +299,63 @@ def test_flash_attn_masked_tiles(block, d, bias_dtype, dtype):
     assert torch.all(dk[dead] == 0) and torch.all(dv[dead] == 0)
 
 
+QUEUED_PATTERNS = ["block_causal_128", "block_causal_64", "block_anticausal", "diagonal_band", "random_blocks"]
+QUEUED_CASES = ([(128, 1024, p, s) for p in QUEUED_PATTERNS for s in ("cube", "batch", "static", "cube_fp32")] +
+                [(96, 1024, p, "batch") for p in QUEUED_PATTERNS] + [(128, 1000, p, "cube") for p in QUEUED_PATTERNS])
+
+
+@pytest.mark.parametrize("dtype", HALF)
+@pytest.mark.parametrize("d,T,pattern,bias_shape", QUEUED_CASES)
+def test_flash_attn_masked_tiles_queued_workgroups(d, T, pattern, bias_shape, dtype):
+    """A launch with more workgroups than the chip holds at once first looks for the all -inf tiles at the end (forward,
+    dQ) or the start (dK/dV) of each workgroup's loop and leaves them out of it; smaller launches do not.  Block-shaped
+    masks in a launch of that size (12 x 8 heads x 8 row blocks), checked on one batch element against the oracle, and
+    against the same batch element computed alone in a small launch (the tiles left out contribute exactly nothing:
+    same bits, unless the small launch splits its workgroups along the keys)."""
+    from rgd_triton_amd import flash_attn_func
+
+    g = gen(21)
+    B, H, b0 = 12, 8, 7
+    q, k, v, do = (randn(g, B, T, H, d, dtype=dtype) for _ in range(4))
+    shape = {"cube": (B, H, T, T), "cube_fp32": (B, H, T, T), "batch": (B, 1, T, T), "static": (1, 1, T, T)}[bias_shape]
+    bias = 0.5 * torch.randn(shape, generator=g)
+    i = torch.arange(T)
+    if pattern == "block_causal_128":
+        mask = (i[None, :] // 128) > (i[:, None] // 128)
+    elif pattern == "block_causal_64":
+        mask = (i[None, :] // 64) > (i[:, None] // 64)
+    elif pattern == "block_anticausal":  # the first keys are the hidden ones
+        mask = (i[None, :] // 128) < (i[:, None] // 128)
+    elif pattern == "diagonal_band":  # hidden tiles at both ends of every loop
+        mask = ((i[None, :] // 128) - (i[:, None] // 128)).abs() > 1
+    else:
+        vis = torch.rand(shape[0], shape[1], (T + 127) // 128, (T + 127) // 128, generator=g) < 0.35
+        vis[..., 3] = True
+        mask = ~vis[:, :, i // 128][:, :, :, i // 128]
+    bias = bias.masked_fill(mask, float("-inf")).to(torch.float32 if bias_shape == "cube_fp32" else dtype)
+    qg, kg, vg, dog = to_gpu(q, k, v, do)
+    bg = bias.cuda()
+
+    def run(sl):
+        qs, ks, vs = (t[sl].detach().requires_grad_(True) for t in (qg, kg, vg))
+        bs = bg if bg.shape[0] == 1 else bg[sl]
+        o, lse = flash_attn_func(qs, ks, vs, bs, False, None, return_lse=True)
+        return (o.detach(), lse.detach()) + torch.autograd.grad(o, (qs, ks, vs), dog[sl])
+
+    big = run(slice(0, B))
+    one = slice(b0, b0 + 1)
+    bias_one = bias if bias.shape[0] == 1 else bias[one]
+    ref = reference(q[one], k[one], v[one], bias_one, do[one])
+    if bias_shape == "cube_fp32":  # the low-precision comparison run adds the bias in q's dtype
+        ref = ref[:3] + reference(q[one], k[one], v[one], bias_one.to(dtype), do[one])[3:]
+    check(tuple(t[one] for t in big), ref, T, grad_mult=3, grad_add=2e-3 if bias_shape == "cube_fp32" else 0.0,
+          name=f"{pattern} in a queued launch")
+    small = run(one)
+    for a, b_, n in zip(big, small, ("o", "lse", "dq", "dk", "dv")):
+        a = a[one].float()
+        assert (a - b_.float()).nan_to_num(posinf=0.0, neginf=0.0).abs().max().item() <= 2e-3 * max(1.0, b_.float().nan_to_num(posinf=0.0, neginf=0.0).abs().max().item()), n
+
+
 def test_flash_attn_fully_masked_row_gives_zero():
     g = gen(7)
     q, k, v = (randn(g, 1, 70, 2, 32, dtype=torch.float16) for _ in range(3))
