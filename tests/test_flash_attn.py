@@ -309,13 +309,13 @@ QUEUED_CASES = ([(128, 1024, p, s) for p in QUEUED_PATTERNS for s in ("cube", "b
 def test_flash_attn_masked_tiles_queued_workgroups(d, T, pattern, bias_shape, dtype):
     """A launch with more workgroups than the chip holds at once first looks for the all -inf tiles at the end (forward,
     dQ) or the start (dK/dV) of each workgroup's loop and leaves them out of it; smaller launches do not.  Block-shaped
-    masks in a launch of that size (12 x 8 heads x 8 row blocks), checked on one batch element against the oracle, and
+    masks in a launch of that size (24 x 4 heads x 8 row blocks), checked on one batch element against the oracle, and
     against the same batch element computed alone in a small launch (the tiles left out contribute exactly nothing:
     same bits, unless the small launch splits its workgroups along the keys)."""
     from rgd_triton_amd import flash_attn_func
 
     g = gen(21)
-    B, H, b0 = 12, 8, 7
+    B, H, b0 = 24, 4, 13
     q, k, v, do = (randn(g, B, T, H, d, dtype=dtype) for _ in range(4))
     shape = {"cube": (B, H, T, T), "cube_fp32": (B, H, T, T), "batch": (B, 1, T, T), "static": (1, 1, T, T)}[bias_shape]
     bias = 0.5 * torch.randn(shape, generator=g)
