@@ -312,11 +312,11 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
         RGD_REQUIRE(grid < (1ll << 31), RGD_ERR_UNSUPPORTED, "%s: grid too large", name);
         rc = dtype == RGD_F16 ? dispatch_bwd<f16_t, true>(p, (unsigned)grid, s) : dispatch_bwd<bf16_t, true>(p, (unsigned)grid, s);
         if (rc != RGD_OK) return rc;
-            if (plan.s > 1) {
+        if (plan.s > 1) {
             const unsigned n = (unsigned)plan.items_split(items);
             rc = dtype == RGD_F16 ? dispatch_bwd_merge<f16_t>(p, n, 1, s) : dispatch_bwd_merge<bf16_t>(p, n, 1, s);
             if (rc != RGD_OK) return rc;
-                }
+        }
     }
     if (Tk > 0) {  // dK and dV (reads delta)
         p.nblk = (int)((Tk + BWD_BM - 1) / BWD_BM);
@@ -333,11 +333,11 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
         RGD_REQUIRE(grid < (1ll << 31), RGD_ERR_UNSUPPORTED, "%s: grid too large", name);
         rc = dtype == RGD_F16 ? dispatch_bwd<f16_t, false>(p, (unsigned)grid, s) : dispatch_bwd<bf16_t, false>(p, (unsigned)grid, s);
         if (rc != RGD_OK) return rc;
-            if (plan.s > 1) {
+        if (plan.s > 1) {
             const unsigned n = (unsigned)plan.items_split(items);
             rc = dtype == RGD_F16 ? dispatch_bwd_merge<f16_t>(p, n, 2, s) : dispatch_bwd_merge<bf16_t>(p, n, 2, s);
             if (rc != RGD_OK) return rc;
-                }
+        }
     }
     return RGD_OK;
 }
