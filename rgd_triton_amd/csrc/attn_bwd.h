@@ -133,12 +133,12 @@ __device__ __forceinline__ void store_row16(T* row, int col, int D, bool vec, co
 // ------------------------------------------------------------------------------------------------
 #ifndef RGD_DQ_BN128
 #define RGD_DQ_BN128 32
+#endif
 #ifndef RGD_DQ_TRIM
 #define RGD_DQ_TRIM 1
 #endif
 #ifndef RGD_DQ_SKIP_EARLY
 #define RGD_DQ_SKIP_EARLY 1
-#endif
 #endif
 // 1: the main loop of the dQ kernel without bias (d <= 64) fetches two tiles ahead
 #ifndef RGD_DQ_PREFETCH2
