@@ -246,7 +246,10 @@ enum rgd_attn_bwd_mode { RGD_ATTN_BWD_AUTO = 0, RGD_ATTN_BWD_TWO_KERNEL = 1, RGD
 /* bytes of scratch for rgd_attn_bwd in the given mode (any contents on entry, 16-byte aligned): delta, fp32
  * (B,H,Tq_rounded), which is required; for the one-pass form dq_accum, fp32 (B,H,Tq_rounded,D padded to 32 or 64),
  * required by RGD_ATTN_BWD_ONE_PASS; then room for the fp32 partial sums of split workgroups (as in
- * rgd_attn_fwd_workspace), which is optional: a smaller workspace is accepted and nothing is split. */
+ * rgd_attn_fwd_workspace), which is optional: a smaller workspace is accepted and nothing is split; and, for head dims
+ * above 64, two ints for every 32 query rows in which the dQ launch tells the dK/dV launch which keys those rows
+ * see through a bias with -inf blocks (optional as well: without room for them the dK/dV launch looks at the bias
+ * itself, with the same results). */
 size_t rgd_attn_bwd_workspace(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, int mode);
 
 /* replaces _flash_attn_backward, flash_attn/flash_attn_triton_cached.py:885-1075

@@ -46,6 +46,11 @@ size_t fwd_part_bytes(int dpad) { return (size_t)ATTN_BM * dpad * sizeof(float) 
 int bwd_blocks_per_cu(int dpad) { return dpad <= 64 ? 2 : 1; }           // dK/dV kernel
 int dq_blocks_per_cu(int dpad) { return (dpad <= 64 || dpad == 128) ? 2 : 1; }  // dQ kernel (32-key tiles at 128)
 size_t bwd_part_bytes(int dpad, int tensors) { return (size_t)tensors * BWD_BM * dpad * sizeof(float); }
+// key ranges the dQ launch leaves for the dK/dV launch (head dims above 64): two ints for every 32 query rows
+int64_t bwd_rows32(int64_t Tq) { return (Tq + BWD_BM - 1) / BWD_BM * (BWD_BM / 32); }  // whole row blocks of the dQ launch
+size_t bwd_ranges_bytes(int64_t B, int64_t H, int64_t Tq, int dpad) {
+    return dpad > 64 ? (size_t)(B * H * bwd_rows32(Tq)) * 2 * sizeof(int) : 0;
+}
 size_t bwd_delta_bytes(int64_t B, int64_t H, int64_t Tq) { return (size_t)(B * H * rgd_attn_seqlen_q_rounded(Tq)) * sizeof(float); }
 // one-pass form: fp32 dq_accum (B, H, Tq_rounded, DPAD) behind delta
 size_t bwd_accum_bytes(int64_t B, int64_t H, int64_t Tq, int dpad) { return bwd_delta_bytes(B, H, Tq) * (size_t)dpad; }
@@ -178,7 +183,7 @@ size_t rgd_attn_bwd_workspace(int64_t B, int64_t H, int64_t Tq, int64_t, int64_t
     const int dpad = attn_dpad(D < 1 ? 1 : D);
     const bool accum = mode != RGD_ATTN_BWD_TWO_KERNEL && D <= 64 && (mode == RGD_ATTN_BWD_ONE_PASS || RGD_ATTN_BWD_AUTO_ONE_PASS);
     return bwd_delta_bytes(B, H, Tq) + (accum ? bwd_accum_bytes(B, H, Tq, dpad) : 0) +
-           (size_t)2 * rgd_num_cus() * bwd_blocks_per_cu(dpad) * bwd_part_bytes(dpad, 2);
+           (size_t)2 * rgd_num_cus() * bwd_blocks_per_cu(dpad) * bwd_part_bytes(dpad, 2) + bwd_ranges_bytes(B, H, Tq, dpad) + 16;
 }
 
 int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const rgd_tensor4* dout, const rgd_tensor4* q,
@@ -227,7 +232,18 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
     const size_t fixed_bytes = delta_bytes + (one_pass ? accum_bytes : 0);
     const bool may_split = workspace && rgd_aligned16(workspace) && !causal;
     float* part_base = reinterpret_cast<float*>(static_cast<char*>(workspace) + fixed_bytes);
-    const size_t part_room = workspace_bytes - fixed_bytes;
+    size_t part_room = workspace_bytes - fixed_bytes;
+    // With a bias at head dims above 64 the dQ launch notes, per 32 query rows, the keys whose bias is above -inf, and the
+    // dK/dV launch starts every key block at the first rows that have such keys (a block-causal bias: half of its loop).
+    // The notes live at the end of the workspace when it has room for them.
+    int* ranges = nullptr;
+    const size_t ranges_bytes = bwd_ranges_bytes(B, H, Tq, dpad);
+    if (!one_pass && !want_dbias && !causal && bias_kind != RGD_BIAS_NONE && dpad > 64 && Tq > 0 && Tk > 0 && workspace &&
+        workspace_bytes >= fixed_bytes + ranges_bytes + 16) {
+        const size_t tail = (workspace_bytes - ranges_bytes) & ~(size_t)15;
+        ranges = reinterpret_cast<int*>(static_cast<char*>(workspace) + tail);
+        part_room = tail - fixed_bytes;
+    }
     const int per_cu = one_pass ? RGD_FUSED_OCC : bwd_blocks_per_cu(dpad);
 
     AttnBwdParams p;
@@ -307,6 +323,8 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
         p.split_full = plan.full;
         p.split_s = plan.s;
         p.trim = items > (int64_t)rgd_num_cus() * dq_blocks_per_cu(dpad);  // see rgd_attn_fwd
+        p.ranges = ranges;
+        p.nrows32 = (int)bwd_rows32(Tq);
         p.part = part_base;
         const int64_t grid = plan.blocks(items);
         RGD_REQUIRE(grid < (1ll << 31), RGD_ERR_UNSUPPORTED, "%s: grid too large", name);
@@ -328,6 +346,8 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
         p.split_full = plan.full;
         p.split_s = plan.s;
         p.trim = items > (int64_t)rgd_num_cus() * per_cu;
+        p.ranges = ranges;
+        p.nrows32 = (int)bwd_rows32(Tq);
         p.part = part_base;
         const int64_t grid = plan.blocks(items);
         RGD_REQUIRE(grid < (1ll << 31), RGD_ERR_UNSUPPORTED, "%s: grid too large", name);

@@ -52,6 +52,11 @@ struct AttnBwdParams {
     int split_full, split_s;
     int group_lg;  // dQ launch: see row_block_of
     int trim;      // this launch looks for leading (dK/dV) or trailing (dQ) all -inf bias tiles first
+    // Key ranges seen by the dQ launch, read by the dK/dV launch of the same call (or null): for every 32 query rows
+    // (B * H * nrows32 entries of two ints) the first key and the end of the last key of the 32-key blocks in which some
+    // pair of those rows had a bias above -inf.  Outside that range P = 0 for those rows.
+    int* ranges;
+    int nrows32;   // entries per (batch, head): 4 * ceil(Tq / 128)
     float* part;
     float* dq_accum;  // one-pass form: fp32 (B, H, Tq_rounded, DPAD), cleared by attn_bwd_prep_kernel
     // bias gradient (optional, dQ kernel): dS = P * (dP - delta) of every (query, key) pair, in the bias dtype, as a
@@ -315,6 +320,9 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
 
     // One key tile.  FAST: tiles j and j+1 are full tiles on the 16-byte path (and the bias, if any, is aligned).
     // AHEAD 0: the step fetches tile j+1 and stores it at its end.  AHEAD 1 / 2 (j even / odd): it fetches tile j+2
+    // tiles of this wavefront with a bias above -inf somewhere (wavefront-uniform): first, and end of the last
+    constexpr bool RECORD = attn_skip_masked(DPAD, BIAS) && !DBIAS;
+    int live_first = 0x7fffffff, live_end = 0;
     // into the staging set of j's parity and stores tile j+1, fetched by the step before, from the other set.
     auto tile_step = [&](const int j, auto FAST, auto AHEAD) __attribute__((always_inline)) {
         constexpr bool F = decltype(FAST)::value != 0;
@@ -336,6 +344,12 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
 #if RGD_DQ_SKIP_EARLY
         if constexpr (attn_skip_masked(DPAD, BIAS)) masked_tile = bias_cur.all_neg_inf(0, NKB);
 #endif
+        if constexpr (RGD_DQ_SKIP_EARLY && RECORD) {
+            if (!masked_tile) {
+                live_first = min(live_first, j);
+                live_end = j + 1;
+            }
+        }
         // the dP accumulators start from -delta, so that product comes out as dP - delta
         f32x16 s[NKB], dp[NKB];
         if (!masked_tile) {
@@ -361,6 +375,12 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
 #if !RGD_DQ_SKIP_EARLY
         if constexpr (attn_skip_masked(DPAD, BIAS)) masked_tile = bias_cur.all_neg_inf(0, NKB);
 #endif
+        if constexpr (!RGD_DQ_SKIP_EARLY && RECORD) {
+            if (!masked_tile) {
+                live_first = min(live_first, j);
+                live_end = j + 1;
+            }
+        }
         if (!masked_tile) {
         float bias_v[NKB][16];
         if constexpr (HAS_BIAS) bias_cur.decode(bias_v);
@@ -475,6 +495,15 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
         for (; j < t_end; ++j) tile_step(j, IntC<0>{}, IntC<0>{});
     }
 
+    if constexpr (RECORD) {
+        if (p.ranges != nullptr && lane == 0 && item.part == 0) {
+            // a part of a split item has seen a part of the keys: its rows are noted as having all of them
+            const bool whole = item.nparts > 1;
+            int* r = p.ranges + (((int64_t)bh * p.nrows32) + qb * (BWD_BM / 32) + wave) * 2;
+            r[0] = whole ? 0 : (live_end > 0 ? live_first * BN : p.Tk);
+            r[1] = whole ? p.Tk : min(live_end * BN, p.Tk);
+        }
+    }
     if (item.nparts > 1) {  // part of a split item: leave the unscaled fp32 sums
         float* row = p.part + ((int64_t)item.part_id * BWD_BM + wave * 32 + li) * DPAD;
 #pragma unroll
@@ -696,7 +725,7 @@ __global__ __launch_bounds__(BWD_THREADS, dkv_occupancy(DPAD, BIAS, FUSED)) void
     const int ntiles_all = (p.Tq + BQ - 1) / BQ;
     const int tile_first = p.causal ? min(ntiles_all, (kblk * BWD_BM) / BQ) : 0;
     int tile_begin = tile_first + (int)((int64_t)(ntiles_all - tile_first) * item.part / item.nparts);
-    const int ntiles = tile_first + (int)((int64_t)(ntiles_all - tile_first) * (item.part + 1) / item.nparts);
+    int ntiles = tile_first + (int)((int64_t)(ntiles_all - tile_first) * (item.part + 1) / item.nparts);
 
     // Leading query tiles whose bias is -inf for every (query, key) pair of the workgroup give P = 0 and add nothing to dK
     // and dV (a block-causal bias: all queries before the key block).  They are found here, before anything else is
@@ -704,7 +733,33 @@ __global__ __launch_bounds__(BWD_THREADS, dkv_occupancy(DPAD, BIAS, FUSED)) void
     // a time, 16 bytes per lane, until it meets a value above -inf; the workgroup starts at the earliest such step.
     // (Inside the loop such a step still costs its tile loads, its first two products and a barrier.)
     if constexpr (attn_skip_masked(DPAD, BIAS) && !FUSED && RGD_DKV_SKIP_PREFIX) {
-        if (p.trim && p.bias_vec && !p.causal && (kblk + 1) * BWD_BM <= p.Tk && tile_begin < ntiles) {
+        if (p.ranges != nullptr && !p.causal && tile_begin < ntiles) {
+            // the dQ launch of this call has left, for every 32 query rows, the range of keys with a bias above -inf:
+            // the first and the last step that have such rows for this key block, without reading the bias
+            constexpr int PER = BQ / 32;
+            const int* rg = p.ranges + (int64_t)bh * p.nrows32 * 2;
+            const int k0 = kblk * BWD_BM, k1 = min(p.Tk, k0 + BWD_BM);
+            int* slot = reinterpret_cast<int*>(smem_raw);
+            if (tid == 0) {
+                slot[0] = ntiles;      // first live step
+                slot[1] = tile_begin;  // end of the last live step
+            }
+            __syncthreads();
+            const int r_end = min(ntiles * PER, p.nrows32);
+            for (int r0 = tile_begin * PER; r0 < r_end; r0 += BWD_THREADS) {
+                const int r = r0 + tid;
+                const bool live = r < r_end && rg[2 * r] < k1 && rg[2 * r + 1] > k0;
+                const uint64_t m = __builtin_amdgcn_ballot_w64(live);
+                if (m != 0 && lane == 0) {
+                    atomicMin(&slot[0], (r + (int)__builtin_ctzll(m)) / PER);
+                    atomicMax(&slot[1], (r + 63 - (int)__builtin_clzll(m)) / PER + 1);
+                }
+            }
+            __syncthreads();
+            tile_begin = max(tile_begin, slot[0]);
+            ntiles = min(ntiles, max(slot[1], tile_begin));
+            __syncthreads();  // the tile buffers are written next
+        } else if (p.trim && p.bias_vec && !p.causal && (kblk + 1) * BWD_BM <= p.Tk && tile_begin < ntiles) {
             constexpr int EPC = 16 / (int)sizeof(TB);  // bias elements per 16 bytes
             constexpr int CPW = 32 / EPC;              // 16-byte chunks of the wavefront's 32 keys in a row
             constexpr int RPL = 64 / CPW;              // rows per load instruction

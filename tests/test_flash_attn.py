@@ -356,6 +356,97 @@ def test_flash_attn_masked_tiles_queued_workgroups(d, T, pattern, bias_shape, dt
         assert (a - b_.float()).nan_to_num(posinf=0.0, neginf=0.0).abs().max().item() <= 2e-3 * max(1.0, b_.float().nan_to_num(posinf=0.0, neginf=0.0).abs().max().item()), n
 
 
+@pytest.mark.parametrize("dtype", HALF)
+@pytest.mark.parametrize("bias_shape", ["cube", "batch", "vector"])
+@pytest.mark.parametrize("pattern", ["block_causal", "block_anticausal", "band", "random_blocks", "none_hidden", "all_hidden_rows"])
+@pytest.mark.parametrize("d,Tq,Tk", [(128, 700, 520), (96, 384, 640), (128, 128, 1024), (128, 1100, 96)])
+def test_flash_attn_bwd_key_ranges(d, Tq, Tk, pattern, bias_shape, dtype):
+    """With room in the workspace, the dQ launch of rgd_attn_bwd notes which keys each 32 query rows can see (bias above
+    -inf) and the dK/dV launch leaves the query tiles before the first and after the last such rows out of each key
+    block's loop.  Through the C ABI: a workspace with room for delta and the notes only (no split), the full workspace
+    (split items note all keys) and a workspace without room for the notes must give the same dK and dV bit for bit
+    (the steps left out add exact zeros), and the oracle's values."""
+    import ctypes
+    from rgd_triton_amd import _hip
+
+    lib = _hip.lib()
+    g = gen(31)
+    B, H = 2, 3
+    q, do = randn(g, B, Tq, H, d, dtype=dtype), randn(g, B, Tq, H, d, dtype=dtype)
+    k, v = randn(g, B, Tk, H, d, dtype=dtype), randn(g, B, Tk, H, d, dtype=dtype)
+    shape = {"cube": (B, H, Tq, Tk), "batch": (B, 1, Tq, Tk), "vector": (B, H, 1, Tk)}[bias_shape]
+    bias = 0.5 * torch.randn(shape, generator=g)
+    qi, ki = torch.arange(shape[2])[:, None] // 64, torch.arange(Tk)[None, :] // 64
+    qs = qi * ((Tk + 63) // 64) // ((Tq + 63) // 64)  # the row block's place on the key axis: every row sees some key
+    if pattern == "block_causal":
+        mask = ki > qs
+    elif pattern == "block_anticausal":
+        mask = ki < qs - 1
+    elif pattern == "band":
+        mask = (ki - qs).abs() > 1
+    elif pattern == "random_blocks":
+        vis = torch.rand(shape[0], shape[1], (shape[2] + 63) // 64, (Tk + 63) // 64, generator=g) < 0.3
+        vis[..., 1] = True
+        mask = ~vis[:, :, torch.arange(shape[2]) // 64][:, :, :, torch.arange(Tk) // 64]
+    elif pattern == "none_hidden":
+        mask = torch.zeros(shape[2], Tk, dtype=torch.bool)
+    else:  # whole row blocks see nothing, the others everything
+        mask = ((qi % 3) == 1).expand(shape[2], Tk)
+    if bias_shape == "vector":  # a vector can only hide keys from every query
+        mask = (ki % 3 == 1) if pattern not in ("none_hidden",) else torch.zeros(1, Tk, dtype=torch.bool)
+    bias = bias.masked_fill(mask, float("-inf")).to(dtype)
+    qg, kg, vg, dog, bg = (t.cuda() for t in (q, k, v, do, bias))
+    code = _hip.dtype_code(dtype)
+    be = bg.expand(B, H, Tq, Tk)
+    kind = _hip.BIAS_VECTOR if bias_shape == "vector" else _hip.BIAS_MATRIX
+    bdesc = _hip.Tensor4(be.data_ptr(), be.stride(0), be.stride(1), be.stride(2))
+    st = _hip.stream_ptr(qg.device)
+    scale = 1.0 / math.sqrt(d)
+    tqr = lib.rgd_attn_seqlen_q_rounded(Tq)
+    delta_bytes = B * H * tqr * 4
+    notes_bytes = B * H * ((Tq + 127) // 128) * 4 * 2 * 4
+    full_b = lib.rgd_attn_bwd_workspace(B, H, Tq, Tk, d, 1)
+    assert full_b >= delta_bytes + notes_bytes + 16
+    o = torch.empty_like(qg)
+    lse = torch.empty(B, H, tqr, dtype=torch.float32, device="cuda")
+    t = {n: _hip.t4(x, False) for n, x in dict(q=qg, k=kg, v=vg, do=dog, o=o).items()}
+    assert lib.rgd_attn_fwd(B, H, Tq, Tk, d, t["q"], t["k"], t["v"], bdesc, kind, code, t["o"], lse.data_ptr(), code, 0, scale,
+                            None, 0, st) == 0, lib.rgd_last_error()
+
+    def run(bws_bytes):
+        dq, dk, dv = torch.empty_like(qg), torch.empty_like(kg), torch.empty_like(vg)
+        bws = torch.empty(bws_bytes, dtype=torch.uint8, device="cuda")
+        tt = {n: _hip.t4(x, False) for n, x in dict(dq=dq, dk=dk, dv=dv).items()}
+        rc = lib.rgd_attn_bwd(B, H, Tq, Tk, d, t["do"], t["q"], t["k"], t["v"], t["o"], lse.data_ptr(), bdesc, kind, code,
+                              tt["dq"], tt["dk"], tt["dv"], None, code, 0, scale, 1, bws.data_ptr(), bws_bytes, st)
+        assert rc == 0, lib.rgd_last_error()
+        torch.cuda.synchronize()
+        return dq, dk, dv
+
+    plain = run(delta_bytes)                       # no notes, no split
+    noted = run(delta_bytes + notes_bytes + 16)    # notes, no room to split
+    full = run(full_b)                             # notes, and whatever the library splits
+    for a, b_, n in zip(noted, plain, ("dq", "dk", "dv")):
+        assert torch.equal(a, b_), f"{n} differs when the dK/dV launch uses the noted key ranges"
+    ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+    for a, b_, n in zip(full, plain, ("dq", "dk", "dv")):
+        assert maxdiff(a, b_.cpu()) <= 1.01 * ulp * max(b_.float().abs().max().item(), 1.0), n
+    g_ref = oracle.attention_bwd(do, q, k, v, bias, False, None)
+    for a, n in zip(noted, ("dq", "dk", "dv")):
+        assert not torch.isnan(a).any(), n
+    if pattern == "all_hidden_rows" and bias_shape != "vector":
+        # the low-precision PyTorch run gives NaN for a row that sees nothing: absolute bound instead
+        hidden = ((torch.arange(Tq) // 64) % 3) == 1
+        assert torch.all(noted[0][:, hidden.cuda()] == 0)
+        for a, r, n in zip(noted, g_ref, ("dq", "dk", "dv")):
+            assert maxdiff(a, r) <= ABS_HALF_ULPS * half_ulp(dtype) * max(1.0, r.float().abs().max().item()), n
+        return
+    ql, kl, vl = (x.clone().requires_grad_(True) for x in (q, k, v))
+    g_pt = torch.autograd.grad(oracle.attention_lowp(ql, kl, vl, bias, False), (ql, kl, vl), do)
+    for a, r, pt, n in zip(noted, g_ref, g_pt, ("dq", "dk", "dv")):
+        assert maxdiff(a, r) <= 3 * maxdiff(pt, r) + 1e-5, f"{n}: {maxdiff(a, r)} vs {maxdiff(pt, r)}"
+
+
 def test_flash_attn_fully_masked_row_gives_zero():
     g = gen(7)
     q, k, v = (randn(g, 1, 70, 2, 32, dtype=torch.float16) for _ in range(3))
