@@ -8,7 +8,7 @@ import math
 import pytest
 import torch
 
-from helpers import assert_repeats_bit_exact, gen, oracle, randn, to_gpu
+from helpers import assert_repeats_bit_exact, gen, gpu_gen, oracle, randn, to_gpu
 
 pytestmark = pytest.mark.gpu
 
@@ -472,7 +472,7 @@ def test_flash_attn_race_condition(Tq, Tk, bias_type, d):
     move by rounding noise (:368,383); here o, lse, dq, dk and dv must all reproduce bit for bit."""
     from rgd_triton_amd import flash_attn_func
 
-    g = gen(8)
+    g = gpu_gen(8)
     dtype = torch.float16
     B, H = 60, 4
     q, k, v = randn(g, B, Tq, H, d, dtype=dtype), randn(g, B, Tk, H, d, dtype=dtype), randn(g, B, Tk, H, d, dtype=dtype)
@@ -580,7 +580,7 @@ def test_flash_attn_race_condition_one_pass(Tq, Tk, bias_type, d, one_pass):
     the rounding noise the reference allows, atol = 2 * max|(dq + 0.3 - 0.3) - dq|."""
     from rgd_triton_amd import flash_attn_func
 
-    g = gen(8)
+    g = gpu_gen(8)
     dtype = torch.float16
     B, H = 60, 4
     q, k, v = randn(g, B, Tq, H, d, dtype=dtype), randn(g, B, Tk, H, d, dtype=dtype), randn(g, B, Tk, H, d, dtype=dtype)

@@ -3,7 +3,7 @@ tests/test_fused_rms.py (parity :139-211, seqdiff with different widths :213-328
 import pytest
 import torch
 
-from helpers import DTYPES, assert_close, assert_repeats_bit_exact, gen, oracle, randn, to_gpu
+from helpers import DTYPES, assert_close, assert_repeats_bit_exact, gen, gpu_gen, oracle, randn, to_gpu
 
 pytestmark = pytest.mark.gpu
 
@@ -112,12 +112,12 @@ def test_fused_rms_norm_race_condition(T1, T2, C, dfactor, unique_bw, dtype):
     of its nine widths and two of its five width ratios; every output and gradient must reproduce bit for bit."""
     from rgd_triton_amd import triton_fused_rms_func_fn
 
-    g = gen(13)
+    g = gpu_gen(13)
     B, C2 = 60, max(1, int(C * (1 + dfactor)))
     x1, x2 = randn(g, B, T1, C, dtype=dtype), randn(g, B, T2, C2, dtype=dtype)
-    w1 = (1 + 0.1 * torch.randn((B, 1, C) if unique_bw else (C,), generator=g)).to(dtype)
-    w2 = (1 + 0.1 * torch.randn((B, 1, C2) if unique_bw else (C2,), generator=g)).to(dtype)
-    d1, d2 = randn(g, B, T1, C, dtype=dtype).cuda(), randn(g, B, T2, C2, dtype=dtype).cuda()
+    w1 = randn(g, *((B, 1, C) if unique_bw else (C,)), dtype=dtype, scale=0.1, shift=1.0)
+    w2 = randn(g, *((B, 1, C2) if unique_bw else (C2,)), dtype=dtype, scale=0.1, shift=1.0)
+    d1, d2 = randn(g, B, T1, C, dtype=dtype), randn(g, B, T2, C2, dtype=dtype)
     a = to_gpu(x1, x2, w1, w2, requires_grad=True)
 
     def step():

@@ -3,7 +3,7 @@ tests/test_head_layernorm.py, tests/test_head_rope.py and tests/test_fused_ln_ro
 import pytest
 import torch
 
-from helpers import DTYPES, assert_close, assert_repeats_bit_exact, gen, oracle, randn, to_gpu
+from helpers import DTYPES, assert_close, assert_repeats_bit_exact, gen, gpu_gen, oracle, randn, to_gpu
 
 pytestmark = pytest.mark.gpu
 
@@ -220,7 +220,7 @@ def test_head_ln_race_condition(Tq, Tk, D, heads_second, dtype):
     """The reference's race test at its own strength (tests/test_head_layernorm.py:214-): batch 60, 4 heads, 250 repeats"""
     from rgd_triton_amd import triton_fused_ln_func_fn
 
-    g = gen(6)
+    g = gpu_gen(6)
     q, k = _qk(g, 60, 4, Tq, Tk, D, dtype, heads_second)
     gq, gk = (t.cuda() for t in _qk(g, 60, 4, Tq, Tk, D, dtype, heads_second))
     qg, kg = to_gpu(q, k, requires_grad=True)
@@ -242,7 +242,7 @@ def test_rope_race_condition(Tq, Tk, D, R, heads_second, dtype, which):
     repeats, on two of their (head dim, rotary dim) combinations; cutoffs inside both sequences."""
     from rgd_triton_amd import triton_fused_ln_rope_fn, triton_rope_fn
 
-    g = gen(6)
+    g = gpu_gen(6)
     q, k = _qk(g, 60, 4, Tq, Tk, D, dtype, heads_second)
     gq, gk = (t.cuda() for t in _qk(g, 60, 4, Tq, Tk, D, dtype, heads_second))
     pe = oracle.rotary_table(max(Tq, Tk) + 1, R, dtype=dtype).to("cuda")

@@ -3,7 +3,7 @@ tests/test_l2normalize.py and tests/test_fused_l2normalize.py (inputs scaled x10
 import pytest
 import torch
 
-from helpers import DTYPES, assert_close, assert_close_allow_inf, assert_repeats_bit_exact, gen, oracle, randn, to_gpu
+from helpers import DTYPES, assert_close, assert_close_allow_inf, assert_repeats_bit_exact, gen, gpu_gen, oracle, randn, to_gpu
 
 pytestmark = pytest.mark.gpu
 
@@ -104,7 +104,7 @@ def test_l2_norm_race_condition(T, C, dtype):
     """The race test of tests/test_l2normalize.py: batch 60, its 9 widths, 250 repeats (three of its eight lengths)"""
     from rgd_triton_amd import triton_norm_func_fn
 
-    g = gen(4)
+    g = gpu_gen(4)
     x = randn(g, 60, T, C, dtype=dtype)
     dy = randn(g, 60, T, C, dtype=dtype).cuda()
     xg = to_gpu(x, requires_grad=True)

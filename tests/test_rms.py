@@ -3,7 +3,7 @@ Counterpart of the reference's tests/test_rms.py (parity :126-184, race :188-246
 import pytest
 import torch
 
-from helpers import DTYPES, assert_close, assert_repeats_bit_exact, gen, oracle, randn, to_gpu
+from helpers import DTYPES, assert_close, assert_repeats_bit_exact, gen, gpu_gen, oracle, randn, to_gpu
 
 pytestmark = pytest.mark.gpu
 
@@ -137,9 +137,9 @@ def test_rms_deterministic_wide(C, T, dtype):
 def _race(B, T, C, dtype, unique_bw):
     from rgd_triton_amd import triton_rms_func_fn
 
-    g = gen(7)
+    g = gpu_gen(7)
     x = randn(g, B, T, C, dtype=dtype, shift=0.5)
-    w = (1 + 0.1 * torch.randn((B, 1, C) if unique_bw else (C,), generator=g)).to(dtype)
+    w = randn(g, *((B, 1, C) if unique_bw else (C,)), dtype=dtype, scale=0.1, shift=1.0)
     dy = randn(g, B, T, C, dtype=dtype)
     xg, wg = to_gpu(x, w, requires_grad=True)
     dyg = dy.to("cuda")
