@@ -168,15 +168,24 @@ template <typename TB, int NKB = 2> struct BiasRuns {
 // above -inf; the workgroup keeps the tiles up to the latest such tile.  (Inside the loop such a tile still costs its
 // K/V loads and a barrier.)  wave_rows: &bias[b, h, first row of the wavefront, 0]; rows: how many of its 32 rows exist;
 // slot: an int in LDS that nothing else uses until the next barrier after the call.  All tiles must be full tiles.
+// A first look that is the same in every wavefront keeps an ordinary bias cheap: the first four bytes of the last tile in
+// each of the workgroup's rows (wg_rows: &bias[b, h, first row of the workgroup, 0], wg_nrows of them, at most 128); one
+// value above -inf there and the last tile stays, with no search and no barrier.
 template <typename TB, int BN>
-__device__ __forceinline__ int bias_trim_end(const TB* __restrict__ wave_rows, int64_t sn, int rows, int t_begin, int t_end, int lane,
-                                             int tid, int* slot) {
+__device__ __forceinline__ int bias_trim_end(const TB* __restrict__ wg_rows, int wg_nrows, const TB* __restrict__ wave_rows,
+                                             int64_t sn, int rows, int t_begin, int t_end, int lane, int tid, int* slot) {
     constexpr int EPC = 16 / (int)sizeof(TB);
     constexpr int CPR = BN / EPC;   // 16-byte chunks per row of a tile
     constexpr int RPL = 64 / CPR;   // rows per load instruction
     constexpr int LPT = 32 / RPL;   // load instructions per tile
     constexpr int BATCH = 4;
     constexpr uint32_t PAT = NegInfBits<TB>::value;
+    {
+        const TB* last = wg_rows + (int64_t)(t_end - 1) * BN;
+        const uint32_t a = *reinterpret_cast<const uint32_t*>(last + (int64_t)min(lane, wg_nrows - 1) * sn);
+        const uint32_t c = *reinterpret_cast<const uint32_t*>(last + (int64_t)min(lane + 64, wg_nrows - 1) * sn);
+        if (__builtin_amdgcn_ballot_w64(a != PAT || c != PAT) != 0) return t_end;  // the same answer in every wavefront
+    }
     int last = t_begin;  // end of this wavefront's live tiles
     if (rows > 0) {
         const TB* col = wave_rows + (lane % CPR) * EPC;

@@ -140,8 +140,10 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
     if constexpr (attn_skip_masked(DPAD, BIAS) && RGD_FWD_TRIM) {
         if (p.trim && p.bias_vec && !p.causal && p.Tk % ATTN_BN == 0 && t_begin < t_end) {
             const int row0 = qb * ATTN_BM + __builtin_amdgcn_readfirstlane(wave) * 32;
-            const TB* rows = static_cast<const TB*>(p.bias.ptr) + b * p.bias.sb + h * p.bias.sh + (int64_t)min(row0, p.Tq - 1) * p.bias.sn;
-            t_end = bias_trim_end<TB, ATTN_BN>(rows, p.bias.sn, min(32, p.Tq - row0), t_begin, t_end, lane, tid,
+            const TB* bh_rows = static_cast<const TB*>(p.bias.ptr) + b * p.bias.sb + h * p.bias.sh;
+            const TB* rows = bh_rows + (int64_t)min(row0, p.Tq - 1) * p.bias.sn;
+            t_end = bias_trim_end<TB, ATTN_BN>(bh_rows + (int64_t)(qb * ATTN_BM) * p.bias.sn, min(ATTN_BM, p.Tq - qb * ATTN_BM), rows,
+                                               p.bias.sn, min(32, p.Tq - row0), t_begin, t_end, lane, tid,
                                                reinterpret_cast<int*>(smem_raw));
         }
     }
