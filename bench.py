@@ -315,6 +315,12 @@ def attention_case(torch, name, B, T, H, D, dtype, bias_kind, iters=20, with_cpu
             dead = T - 256 + torch.randperm(256, generator=g)[:26]
             bias[b, :, :, dead] = float("-inf")
         bias = bias.to(dtype).cuda()
+    elif bias_kind == "zero_shared":  # comparison workloads (--only): what the bias of config 5 costs
+        bias = torch.zeros(B, 1, T, T, dtype=dtype, device="cuda")
+    elif bias_kind == "dense_shared":
+        bias = (0.5 * torch.randn(B, 1, T, T, generator=g)).to(dtype).cuda()
+    elif bias_kind == "dense_full":
+        bias = (0.5 * torch.randn(B, H, T, T, generator=g)).to(dtype).cuda()
     o, dq, dk, dv = (torch.empty_like(q) for _ in range(4))
     tqr = lib.rgd_attn_seqlen_q_rounded(T)
     lse = torch.empty(B, H, tqr, dtype=torch.float32, device="cuda")
@@ -330,14 +336,23 @@ def attention_case(torch, name, B, T, H, D, dtype, bias_kind, iters=20, with_cpu
     t = {n: _hip.t4(x, False) for n, x in dict(q=q, k=k, v=v, do=do, o=o, dq=dq, dk=dk, dv=dv).items()}
     st = _hip.stream_ptr(q.device)
     scale = 1.0 / math.sqrt(D)
+    # tile classes of a head-shared bias: written once per step, in the forward (as the autograd Function does), and
+    # passed to both calls; RGD_BENCH_CLASSES=0 passes none and lets each call classify on its own
+    cls_bytes = lib.rgd_attn_bias_classes_bytes(B, H, T, T, D, bdesc, bk, bd) if bias is not None else 0
+    if os.environ.get("RGD_BENCH_CLASSES", "1") == "0":
+        cls_bytes = 0
+    cls_buf = torch.empty(max(cls_bytes, 8) // 8, dtype=torch.int64, device="cuda")
+    cls_ptr = cls_buf.data_ptr() if cls_bytes else None
 
     def fwd():
+        if cls_bytes:
+            assert lib.rgd_attn_bias_classify(B, H, T, T, D, bdesc, bk, bd, cls_ptr, cls_bytes, st) == 0, lib.rgd_last_error()
         assert lib.rgd_attn_fwd(B, H, T, T, D, t["q"], t["k"], t["v"], bdesc, bk, bd, t["o"], lse.data_ptr(), code, 0,
-                                scale, fws.data_ptr(), fws.numel(), st) == 0, lib.rgd_last_error()
+                                scale, cls_ptr, fws.data_ptr(), fws.numel(), st) == 0, lib.rgd_last_error()
 
     def bwd():
         assert lib.rgd_attn_bwd(B, H, T, T, D, t["do"], t["q"], t["k"], t["v"], t["o"], lse.data_ptr(), bdesc, bk, bd,
-                                t["dq"], t["dk"], t["dv"], None, code, 0, scale, mode, ws.data_ptr(), ws.numel(), st) == 0, \
+                                t["dq"], t["dk"], t["dv"], None, code, 0, scale, mode, cls_ptr, ws.data_ptr(), ws.numel(), st) == 0, \
             lib.rgd_last_error()
 
     # forward and backward alternate as in a training step; the clocks are brought to their steady state first
@@ -534,6 +549,16 @@ def extras(torch, only="", with_cpu=False):
     if want("attn_c5"):
         out.append(attention_case(torch, "attn_c5: (2,4352,24,64) bf16 broadcast bias", 2, 4352, 24, 64, bf, "broadcast", with_cpu=with_cpu))
 
+    # comparison workloads, only when named: the config-5 shape without bias, with an all-zero and with a dense head-shared
+    # bias; the config-4 shape with a finite bias (no -inf blocks to leave out)
+    if only == "attn_c5_nobias":
+        out.append(attention_case(torch, "attn_c5_nobias: (2,4352,24,64) bf16 no bias", 2, 4352, 24, 64, bf, None))
+    if only == "attn_c5_zero":
+        out.append(attention_case(torch, "attn_c5_zero: (2,4352,24,64) bf16 (B,1,T,T) bias of zeros", 2, 4352, 24, 64, bf, "zero_shared"))
+    if only == "attn_c5_dense":
+        out.append(attention_case(torch, "attn_c5_dense: (2,4352,24,64) bf16 (B,1,T,T) dense bias", 2, 4352, 24, 64, bf, "dense_shared"))
+    if only == "attn_c4_finite":
+        out.append(attention_case(torch, "attn_c4_finite: (2,2048,16,128) fp16 (B,H,T,T) finite bias", 2, 2048, 16, 128, torch.float16, "dense_full"))
     # buffer sets are sized so that their sum exceeds the 256 MB Infinity Cache
     if want("rms_c1"):
         out.append(rms_case(torch, "rms_c1: FusedRMSNorm (4,1024,1024) fp32 fwd+bwd", 4, [(1024, 1024)], torch.float32, 12, with_cpu=with_cpu))

@@ -214,21 +214,40 @@ int rgd_ln_rope_qk_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D,
  * them (flash_attn/flash_attn_triton_cached.py:790-792) */
 int64_t rgd_attn_seqlen_q_rounded(int64_t Tq);
 
+/* Tile classes of a bias matrix that the heads share (stride_h == 0), head dims up to 64.  Such a bias is usually a
+ * mask (0 / -inf), and the reference streams it tile by tile for every head and in every kernel
+ * (flash_attn/flash_attn_triton_cached.py:151-175, :430-470).  One pass over the matrix leaves two bits per tile of 32
+ * queries x 64 keys (all +0, all -inf, anything else); rgd_attn_fwd and rgd_attn_bwd then run tiles that are all +0
+ * like tiles without bias, leave all -inf tiles out and read the bias only for the others, with the same results bit
+ * for bit.  Both calls make that pass themselves, into the end of their workspace, when bias_classes is NULL; a caller
+ * that runs several calls on one bias (a forward and its backward) can make it once:
+ *   rgd_attn_bias_classes_bytes  size of the classes for this bias and shape; 0 when they would not be used
+ *                                (bias not a matrix, not shared by the heads, rows not 16-byte aligned, D > 64, H < 2)
+ *   rgd_attn_bias_classify       writes them (8-byte aligned buffer of that size), one kernel launch on `stream`
+ * and pass the buffer as bias_classes.  The classes describe the bias VALUES: classify again when they change. */
+size_t rgd_attn_bias_classes_bytes(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D,
+                                   const rgd_tensor4* bias, int bias_kind, int bias_dtype);
+int rgd_attn_bias_classify(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D,
+                           const rgd_tensor4* bias, int bias_kind, int bias_dtype,
+                           void* classes, size_t classes_bytes, void* stream);
+
 /* replaces _flash_attn_forward, flash_attn/flash_attn_triton_cached.py:758-882 (kernel :21-246).
  * lse is fp32 (B, H, Tq_rounded); rows >= Tq are written as 0.  A query row whose logits are all
- * -inf gives o = 0 and lse = -inf. */
+ * -inf gives o = 0 and lse = -inf.  bias_classes: NULL, or what rgd_attn_bias_classify wrote for this bias. */
 int rgd_attn_fwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D,
                  const rgd_tensor4* q, const rgd_tensor4* k, const rgd_tensor4* v,
                  const rgd_tensor4* bias, int bias_kind, int bias_dtype,
                  const rgd_tensor4* o, float* lse,
-                 int dtype, int causal, float softmax_scale,
+                 int dtype, int causal, float softmax_scale, const void* bias_classes,
                  void* workspace, size_t workspace_bytes, void* stream);
 
 /* Optional scratch of rgd_attn_fwd (any contents on entry, 16-byte aligned).  With it, the query blocks of
  * the last, partly filled round of workgroups are split along the keys and merged by a second launch, which
- * fills the chip for grids that are not a multiple of the resident workgroups (and for small grids).
- * workspace = NULL or a smaller buffer is legal: the call then splits less or not at all.  Results do not
- * depend on scheduling; a split item sums its keys in a different grouping than an unsplit one. */
+ * fills the chip for grids that are not a multiple of the resident workgroups (and for small grids).  Its end holds the
+ * tile classes of a head-shared bias when the caller passes none (8-byte aligned workspace).
+ * workspace = NULL or a smaller buffer is legal: the call then splits less or not at all, and reads such a bias like
+ * any other.  Results do not depend on scheduling; a split item sums its keys in a different grouping than an unsplit
+ * one. */
 size_t rgd_attn_fwd_workspace(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D);
 
 /* Forms of the attention backward.
@@ -249,7 +268,8 @@ enum rgd_attn_bwd_mode { RGD_ATTN_BWD_AUTO = 0, RGD_ATTN_BWD_TWO_KERNEL = 1, RGD
  * rgd_attn_fwd_workspace), which is optional: a smaller workspace is accepted and nothing is split; and, for head dims
  * above 64, two ints for every 32 query rows in which the dQ launch tells the dK/dV launch which keys those rows
  * see through a bias with -inf blocks (optional as well: without room for them the dK/dV launch looks at the bias
- * itself, with the same results). */
+ * itself, with the same results); for head dims up to 64, the tile classes of a head-shared bias when the caller passes
+ * none (optional as well). */
 size_t rgd_attn_bwd_workspace(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, int mode);
 
 /* replaces _flash_attn_backward, flash_attn/flash_attn_triton_cached.py:885-1075
@@ -261,14 +281,15 @@ size_t rgd_attn_bwd_workspace(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int6
  * sums over the dimensions its bias broadcasts; with causal != 0 the caller clears it first (key tiles past the
  * diagonal are not visited).  Two-kernel form only.  dq, dk, dv are written
  * in the tensor dtype from fp32 accumulators, each exactly once; in a fixed order except for dq in the one-pass
- * form (see rgd_attn_bwd_mode). */
+ * form (see rgd_attn_bwd_mode).  bias_classes: NULL, or what rgd_attn_bias_classify wrote for this bias (used by the
+ * two-kernel form without a bias gradient). */
 int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D,
                  const rgd_tensor4* dout, const rgd_tensor4* q, const rgd_tensor4* k,
                  const rgd_tensor4* v, const rgd_tensor4* o, const float* lse,
                  const rgd_tensor4* bias, int bias_kind, int bias_dtype,
                  const rgd_tensor4* dq, const rgd_tensor4* dk, const rgd_tensor4* dv,
                  const rgd_tensor4* dbias,
-                 int dtype, int causal, float softmax_scale, int mode,
+                 int dtype, int causal, float softmax_scale, int mode, const void* bias_classes,
                  void* workspace, size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus

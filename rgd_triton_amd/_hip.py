@@ -16,7 +16,7 @@ LIB_PATH = os.environ.get("RGD_HIP_LIB") or os.path.join(_HERE, "librgd_hip.so")
 HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "rgd_hip.h")
 
 RGD_F32, RGD_F16, RGD_BF16 = 0, 1, 2
-ABI_MAJOR = 2  # rgd_version() // 1000 this binding was written for
+ABI_MAJOR = 3  # rgd_version() // 1000 this binding was written for
 BIAS_NONE, BIAS_VECTOR, BIAS_MATRIX = 0, 1, 2
 ATTN_BWD_AUTO, ATTN_BWD_TWO_KERNEL, ATTN_BWD_ONE_PASS = 0, 1, 2
 
@@ -60,11 +60,13 @@ _SIGNATURES = {
     "rgd_ln_rope_qk_bwd": (_int, [_i64] * 5 + [_T4] * 6 + [_vp, _i64, _i64, _i64, _i64, _int, _i64, _i64, _int, _f32,
                                                             _vp]),
     "rgd_attn_seqlen_q_rounded": (_i64, [_i64]),
-    "rgd_attn_fwd": (_int, [_i64] * 5 + [_T4] * 4 + [_int, _int, _T4, _vp, _int, _int, _f32, _vp, _sz, _vp]),
+    "rgd_attn_bias_classes_bytes": (_sz, [_i64] * 5 + [_T4, _int, _int]),
+    "rgd_attn_bias_classify": (_int, [_i64] * 5 + [_T4, _int, _int, _vp, _sz, _vp]),
+    "rgd_attn_fwd": (_int, [_i64] * 5 + [_T4] * 4 + [_int, _int, _T4, _vp, _int, _int, _f32, _vp, _vp, _sz, _vp]),
     "rgd_attn_fwd_workspace": (_sz, [_i64] * 5),
     "rgd_attn_bwd_workspace": (_sz, [_i64] * 5 + [_int]),
     "rgd_attn_bwd": (_int, [_i64] * 5 + [_T4] * 5 + [_vp] + [_T4, _int, _int] + [_T4] * 4 + [_int, _int, _f32, _int, _vp,
-                                                                                         _sz, _vp]),
+                                                                                         _vp, _sz, _vp]),
 }
 
 _lib = None

@@ -6,6 +6,7 @@
 
 // attn_f16.hip / attn_bf16.hip: LDS size attribute of every attention kernel instantiation of one element type
 template <typename T> int attn_configure_all();
+template <typename T> int attn_configure_cls();  // attn_cls_f16.hip / attn_cls_bf16.hip
 // rows_wide.hip: address of the library-owned scratch array on the current device
 int wide_noalloc_setup(void** out);
 
@@ -24,6 +25,8 @@ void init_once() {
         // kernels with more than 48 KB of dynamic LDS need the attribute before their first launch
         rc = attn_configure_all<f16_t>();
         if (rc == RGD_OK) rc = attn_configure_all<bf16_t>();
+        if (rc == RGD_OK) rc = attn_configure_cls<f16_t>();
+        if (rc == RGD_OK) rc = attn_configure_cls<bf16_t>();
         if (rc == RGD_OK) rc = wide_noalloc_setup(nullptr);
     } else {
         // no usable device (a CPU-only process that checks arguments): launches will fail with their own error
@@ -59,7 +62,7 @@ int rgd_launch_status(const char* what, hipError_t e) {
 }
 
 extern "C" {
-int rgd_version(void) { return 2000; }
+int rgd_version(void) { return 3000; }
 const char* rgd_last_error(void) { return g_error; }
 int rgd_init(void) {
     const int rc = rgd_ensure_init();

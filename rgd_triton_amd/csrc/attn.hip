@@ -13,6 +13,12 @@ template <typename T> int dispatch_bwd_merge(const AttnBwdParams& p, unsigned it
 template <typename T, bool DQ> int dispatch_bwd(const AttnBwdParams& p, unsigned grid, hipStream_t s);
 template <typename T> int dispatch_bwd_fused(const AttnBwdParams& p, unsigned grid, hipStream_t s);
 template <typename T> int dispatch_bwd_fused_aux(const AttnBwdParams& p, int which, hipStream_t s);
+// kernels that read the tile classes of a head-shared bias: attn_cls_f16.hip / attn_cls_bf16.hip; the pass that
+// writes the classes: attn_classes.hip
+template <typename T> int dispatch_fwd_cls(const AttnFwdParams& p, unsigned grid, hipStream_t s);
+template <typename T, bool DQ> int dispatch_bwd_cls(const AttnBwdParams& p, unsigned grid, hipStream_t s);
+int attn_classify(const void* bias, int64_t sb, int64_t sn, int bias_dtype, int nb, int64_t Tq, int64_t Tk, uint64_t* words,
+                  hipStream_t s);
 
 // 1: RGD_ATTN_BWD_AUTO takes the one-pass form where it exists
 #ifndef RGD_ATTN_BWD_AUTO_ONE_PASS
@@ -51,6 +57,8 @@ int64_t bwd_rows32(int64_t Tq) { return (Tq + BWD_BM - 1) / BWD_BM * (BWD_BM / 3
 size_t bwd_ranges_bytes(int64_t B, int64_t H, int64_t Tq, int dpad) {
     return dpad > 64 ? (size_t)(B * H * bwd_rows32(Tq)) * 2 * sizeof(int) : 0;
 }
+// dK/dV launches with tile classes: one byte per (batch, key block), see AttnBwdParams::cls_served
+size_t bwd_served_bytes(int64_t B, int64_t Tk) { return ((size_t)(B * ((Tk + BWD_BM - 1) / BWD_BM)) + 15) & ~(size_t)15; }
 size_t bwd_delta_bytes(int64_t B, int64_t H, int64_t Tq) { return (size_t)(B * H * rgd_attn_seqlen_q_rounded(Tq)) * sizeof(float); }
 // one-pass form: fp32 dq_accum (B, H, Tq_rounded, DPAD) behind delta
 size_t bwd_accum_bytes(int64_t B, int64_t H, int64_t Tq, int dpad) { return bwd_delta_bytes(B, H, Tq) * (size_t)dpad; }
@@ -61,6 +69,50 @@ bool bwd_one_pass(int mode, int64_t D, size_t workspace_bytes, size_t need) {
     if (mode == RGD_ATTN_BWD_TWO_KERNEL || D > 64) return false;
     if (mode == RGD_ATTN_BWD_ONE_PASS) return true;
     return RGD_ATTN_BWD_AUTO_ONE_PASS && workspace_bytes >= need;
+}
+
+// Tile classes (attn_classes.h) pay for a bias matrix that several heads share: one pass over it instead of one per
+// head and kernel.  Head dims up to 64 (the kernels for wider heads have no registers for a second code path), rows the
+// 16-byte loads can read, and a key count a wavefront can keep the classes of.
+bool cls_eligible(int64_t H, int64_t Tq, int64_t Tk, int64_t D, const rgd_tensor4* bias, int bias_kind, int bias_dtype) {
+    if (bias_kind != RGD_BIAS_MATRIX || !bias || bias->stride_h != 0 || H < 2 || D > 64 || Tq < 1 || Tk < CLS_KEYS) return false;
+    const int64_t per16 = bias_dtype == RGD_F32 ? 4 : 8;
+    if (!rgd_aligned16(bias->ptr) || bias->stride_b % per16 != 0 || bias->stride_n % per16 != 0) return false;
+    return cls_nwords(Tk) <= CLS_MAX_WORDS && cls_nrow32(Tq) <= CLS_MAX_ROWS;
+}
+int64_t cls_batches(int64_t B, const rgd_tensor4* bias) { return bias->stride_b == 0 ? 1 : B; }
+BiasClasses cls_desc(const void* words, int64_t B, int64_t Tq, int64_t Tk, const rgd_tensor4* bias) {
+    BiasClasses c;
+    c.words = static_cast<const uint64_t*>(words);
+    c.nwords = cls_nwords(Tk);
+    c.nrow32 = cls_nrow32(Tq);
+    c.sb = cls_batches(B, bias) == 1 ? 0 : (int64_t)c.nrow32 * c.nwords;
+    return c;
+}
+// The classes a call works with: the caller's (bias_classes), or written here into the end of the workspace when it has
+// room for them behind `fixed_bytes`; *room is what is left of the workspace in front of them.  Null: none.
+const void* cls_for_call(const char* name, int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const rgd_tensor4* bias,
+                         int bias_kind, int bias_dtype, const void* bias_classes, void* workspace, size_t workspace_bytes,
+                         size_t fixed_bytes, size_t* room, hipStream_t s, int* rc) {
+    *rc = RGD_OK;
+    if (!cls_eligible(H, Tq, Tk, D, bias, bias_kind, bias_dtype)) return nullptr;
+    if (bias_classes) {
+        if ((reinterpret_cast<uintptr_t>(bias_classes) & 7u) != 0) {
+            rgd_set_error("%s: bias_classes must be 8-byte aligned", name);
+            *rc = RGD_ERR_INVALID;
+            return nullptr;
+        }
+        return bias_classes;
+    }
+    const size_t need = cls_bytes(cls_batches(B, bias), Tq, Tk);
+    if (!workspace || workspace_bytes < fixed_bytes + need + 16) return nullptr;
+    const size_t tail = (workspace_bytes - need) & ~(size_t)15;
+    if (reinterpret_cast<uintptr_t>(workspace) & 7u) return nullptr;
+    uint64_t* words = reinterpret_cast<uint64_t*>(static_cast<char*>(workspace) + tail);
+    *rc = attn_classify(bias->ptr, bias->stride_b, bias->stride_n, bias_dtype, (int)cls_batches(B, bias), Tq, Tk, words, s);
+    if (*rc != RGD_OK) return nullptr;
+    *room = tail;
+    return words;
 }
 
 // measured: what a second and third resident workgroup add to a compute unit, and the duration of one inner
@@ -97,15 +149,36 @@ extern "C" {
 
 int64_t rgd_attn_seqlen_q_rounded(int64_t Tq) { return (Tq + 63) / 64 * 64; }
 
-size_t rgd_attn_fwd_workspace(int64_t, int64_t, int64_t, int64_t, int64_t D) {
+size_t rgd_attn_fwd_workspace(int64_t B, int64_t, int64_t Tq, int64_t Tk, int64_t D) {
     if (D < 1 || D > 128) return 0;
-    return (size_t)2 * rgd_num_cus() * 3 * fwd_part_bytes(attn_dpad(D));  // two rounds of parts at the highest occupancy
+    // two rounds of parts at the highest occupancy, then the tile classes of a head-shared bias
+    const size_t cls = (D <= 64 && B > 0 && Tq > 0 && Tk > 0 && cls_nwords(Tk) <= CLS_MAX_WORDS && cls_nrow32(Tq) <= CLS_MAX_ROWS) ? cls_bytes(B, Tq, Tk) + 32 : 0;
+    return (size_t)2 * rgd_num_cus() * 3 * fwd_part_bytes(attn_dpad(D)) + cls;
+}
+
+size_t rgd_attn_bias_classes_bytes(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const rgd_tensor4* bias, int bias_kind,
+                                   int bias_dtype) {
+    if (B < 1 || !cls_eligible(H, Tq, Tk, D, bias, bias_kind, bias_dtype)) return 0;
+    return cls_bytes(cls_batches(B, bias), Tq, Tk);
+}
+
+int rgd_attn_bias_classify(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const rgd_tensor4* bias, int bias_kind,
+                           int bias_dtype, void* classes, size_t classes_bytes, void* stream) {
+    const char* name = "rgd_attn_bias_classify";
+    const int init_rc = rgd_ensure_init();
+    if (init_rc != RGD_OK) return init_rc;
+    const size_t need = rgd_attn_bias_classes_bytes(B, H, Tq, Tk, D, bias, bias_kind, bias_dtype);
+    RGD_REQUIRE(need > 0, RGD_ERR_UNSUPPORTED, "%s: no tile classes for this bias and shape (rgd_attn_bias_classes_bytes is 0)", name);
+    RGD_REQUIRE(classes && (reinterpret_cast<uintptr_t>(classes) & 7u) == 0 && classes_bytes >= need, RGD_ERR_WORKSPACE,
+                "%s: classes needs %zu bytes, 8-byte aligned", name, need);
+    return attn_classify(bias->ptr, bias->stride_b, bias->stride_n, bias_dtype, (int)cls_batches(B, bias), Tq, Tk,
+                         static_cast<uint64_t*>(classes), static_cast<hipStream_t>(stream));
 }
 
 int rgd_attn_fwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const rgd_tensor4* q, const rgd_tensor4* k,
                  const rgd_tensor4* v, const rgd_tensor4* bias, int bias_kind, int bias_dtype, const rgd_tensor4* o,
-                 float* lse, int dtype, int causal, float softmax_scale, void* workspace, size_t workspace_bytes,
-                 void* stream) {
+                 float* lse, int dtype, int causal, float softmax_scale, const void* bias_classes, void* workspace,
+                 size_t workspace_bytes, void* stream) {
     const char* name = "rgd_attn_fwd";
     int rc = check_common(name, B, H, Tq, Tk, D, dtype, bias_kind, bias_dtype, bias);
     if (rc != RGD_OK) return rc;
@@ -147,12 +220,21 @@ int rgd_attn_fwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
                      (p.bias.sn % per16) == 0;
     }
     const int64_t items = (int64_t)p.nqb * B * H;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // tile classes of a head-shared bias: the caller's, or written into the end of the workspace
+    size_t part_room = workspace_bytes;
+    // (not with a softmax scale of 0 or below: the kernels that read classes add the bias in units of the raw scores)
+    const void* cls = softmax_scale > 0.f ? cls_for_call(name, B, H, Tq, Tk, D, bias, bias_kind, bias_dtype, bias_classes, workspace,
+                                                         workspace_bytes, 0, &part_room, s, &rc)
+                                          : nullptr;
+    if (rc != RGD_OK) return rc;
+    if (cls) p.cls = cls_desc(cls, B, Tq, Tk, bias);
     // items of the last, partly filled round are split along the keys when a workspace is given
     const int dpad = attn_dpad(D);
     AttnSplit plan;
     if (workspace && rgd_aligned16(workspace) && !causal)
-        plan = attn_split_plan(items, rgd_num_cus(), fwd_blocks_per_cu(dpad, bias_kind != RGD_BIAS_NONE),
-                               (int)((Tk + ATTN_BN - 1) / ATTN_BN), fwd_part_bytes(dpad), workspace_bytes, kFwdSplit);
+        plan = attn_split_plan(items, rgd_num_cus(), cls ? RGD_CLS_FWD_OCC : fwd_blocks_per_cu(dpad, bias_kind != RGD_BIAS_NONE),
+                               (int)((Tk + ATTN_BN - 1) / ATTN_BN), fwd_part_bytes(dpad), part_room, kFwdSplit);
     p.split_full = plan.full;
     p.split_s = plan.s;
     // Leaving leading / trailing all -inf bias tiles out of a workgroup's loop takes a pass over its bias first.  It pays
@@ -166,7 +248,14 @@ int rgd_attn_fwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
     }
     const int64_t grid = plan.blocks(items);
     RGD_REQUIRE(grid < (1ll << 31), RGD_ERR_UNSUPPORTED, "%s: grid too large", name);
-    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (cls) {
+        // two launches over the same grid: batch elements whose bias is mostly ZERO / NEG tiles run in the variant laid
+        // out like the kernel without bias, the others in the ordinary one (see cls_batch_dense)
+        p.cls_take = 1;
+        rc = dtype == RGD_F16 ? dispatch_fwd_cls<f16_t>(p, (unsigned)grid, s) : dispatch_fwd_cls<bf16_t>(p, (unsigned)grid, s);
+        if (rc != RGD_OK) return rc;
+        p.cls_take = 2;
+    }
     rc = dtype == RGD_F16 ? dispatch_fwd<f16_t>(p, (unsigned)grid, s) : dispatch_fwd<bf16_t>(p, (unsigned)grid, s);
     if (rc != RGD_OK) return rc;
     if (plan.s > 1) {
@@ -177,20 +266,23 @@ int rgd_attn_fwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
     return RGD_OK;
 }
 
-size_t rgd_attn_bwd_workspace(int64_t B, int64_t H, int64_t Tq, int64_t, int64_t D, int mode) {
+size_t rgd_attn_bwd_workspace(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, int mode) {
     // delta, dq_accum where the one-pass form may run, then room for two rounds of dK/dV parts (the dQ parts of the
     // two-kernel form reuse it; the launches are ordered)
     const int dpad = attn_dpad(D < 1 ? 1 : D);
     const bool accum = mode != RGD_ATTN_BWD_TWO_KERNEL && D <= 64 && (mode == RGD_ATTN_BWD_ONE_PASS || RGD_ATTN_BWD_AUTO_ONE_PASS);
+    const size_t cls = (D <= 64 && B > 0 && Tq > 0 && Tk > 0 && cls_nwords(Tk) <= CLS_MAX_WORDS && cls_nrow32(Tq) <= CLS_MAX_ROWS)
+                           ? cls_bytes(B, Tq, Tk) + 32 + bwd_served_bytes(B, Tk)
+                           : 0;
     return bwd_delta_bytes(B, H, Tq) + (accum ? bwd_accum_bytes(B, H, Tq, dpad) : 0) +
-           (size_t)2 * rgd_num_cus() * bwd_blocks_per_cu(dpad) * bwd_part_bytes(dpad, 2) + bwd_ranges_bytes(B, H, Tq, dpad) + 16;
+           (size_t)2 * rgd_num_cus() * bwd_blocks_per_cu(dpad) * bwd_part_bytes(dpad, 2) + bwd_ranges_bytes(B, H, Tq, dpad) + 16 + cls;
 }
 
 int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const rgd_tensor4* dout, const rgd_tensor4* q,
                  const rgd_tensor4* k, const rgd_tensor4* v, const rgd_tensor4* o, const float* lse,
                  const rgd_tensor4* bias, int bias_kind, int bias_dtype, const rgd_tensor4* dq, const rgd_tensor4* dk,
                  const rgd_tensor4* dv, const rgd_tensor4* dbias, int dtype, int causal, float softmax_scale, int mode,
-                 void* workspace, size_t workspace_bytes, void* stream) {
+                 const void* bias_classes, void* workspace, size_t workspace_bytes, void* stream) {
     const char* name = "rgd_attn_bwd";
     RGD_REQUIRE(mode == RGD_ATTN_BWD_AUTO || mode == RGD_ATTN_BWD_TWO_KERNEL || mode == RGD_ATTN_BWD_ONE_PASS,
                 RGD_ERR_INVALID, "%s: bad mode %d", name, mode);
@@ -245,6 +337,24 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
         part_room = tail - fixed_bytes;
     }
     const int per_cu = one_pass ? RGD_FUSED_OCC : bwd_blocks_per_cu(dpad);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // tile classes of a head-shared bias (two-kernel form, no bias gradient): the caller's, or written into the end of
+    // the workspace
+    const void* cls = nullptr;
+    uint8_t* cls_served = nullptr;
+    const size_t served_bytes = bwd_served_bytes(B, Tk);
+    if (!one_pass && !want_dbias && Tq > 0 && Tk > 0 && softmax_scale > 0.f && workspace_bytes >= fixed_bytes + served_bytes) {
+        // the bytes in which the two dK/dV launches agree on who serves a key block sit behind delta
+        size_t tail = workspace_bytes;
+        cls = cls_for_call(name, B, H, Tq, Tk, D, bias, bias_kind, bias_dtype, bias_classes, workspace, workspace_bytes,
+                           fixed_bytes + served_bytes, &tail, s, &rc);
+        if (rc != RGD_OK) return rc;
+        if (cls) {
+            cls_served = reinterpret_cast<uint8_t*>(static_cast<char*>(workspace) + fixed_bytes);
+            part_base = reinterpret_cast<float*>(static_cast<char*>(workspace) + fixed_bytes + served_bytes);
+            part_room = tail - fixed_bytes - served_bytes;
+        }
+    }
 
     AttnBwdParams p;
     memset(&p, 0, sizeof(p));
@@ -282,7 +392,8 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
         p.bias_vec = rgd_aligned16(bias->ptr) && (p.bias.sb % per16) == 0 && (p.bias.sh % per16) == 0 &&
                      (p.bias.sn % per16) == 0;
     }
-    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (cls) p.cls = cls_desc(cls, B, Tq, Tk, bias);
+    p.cls_served = cls_served;
     if (one_pass) {
         p.dq_accum = reinterpret_cast<float*>(static_cast<char*>(workspace) + delta_bytes);
         if (Tq > 0) {  // delta, and dq_accum = 0
@@ -328,6 +439,12 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
         p.part = part_base;
         const int64_t grid = plan.blocks(items);
         RGD_REQUIRE(grid < (1ll << 31), RGD_ERR_UNSUPPORTED, "%s: grid too large", name);
+        if (cls) {  // two launches over the same grid, as in rgd_attn_fwd
+            p.cls_take = 1;
+            rc = dtype == RGD_F16 ? dispatch_bwd_cls<f16_t, true>(p, (unsigned)grid, s) : dispatch_bwd_cls<bf16_t, true>(p, (unsigned)grid, s);
+            if (rc != RGD_OK) return rc;
+            p.cls_take = 2;
+        }
         rc = dtype == RGD_F16 ? dispatch_bwd<f16_t, true>(p, (unsigned)grid, s) : dispatch_bwd<bf16_t, true>(p, (unsigned)grid, s);
         if (rc != RGD_OK) return rc;
         if (plan.s > 1) {
@@ -351,6 +468,12 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
         p.part = part_base;
         const int64_t grid = plan.blocks(items);
         RGD_REQUIRE(grid < (1ll << 31), RGD_ERR_UNSUPPORTED, "%s: grid too large", name);
+        if (cls) {
+            p.cls_take = 1;
+            rc = dtype == RGD_F16 ? dispatch_bwd_cls<f16_t, false>(p, (unsigned)grid, s) : dispatch_bwd_cls<bf16_t, false>(p, (unsigned)grid, s);
+            if (rc != RGD_OK) return rc;
+            p.cls_take = 2;
+        }
         rc = dtype == RGD_F16 ? dispatch_bwd<f16_t, false>(p, (unsigned)grid, s) : dispatch_bwd<bf16_t, false>(p, (unsigned)grid, s);
         if (rc != RGD_OK) return rc;
         if (plan.s > 1) {

@@ -33,6 +33,7 @@
 #pragma once
 
 #include "attn_common.h"
+#include "attn_classes.h"
 
 #include <type_traits>
 
@@ -62,6 +63,14 @@ struct AttnBwdParams {
     // bias gradient (optional, dQ kernel): dS = P * (dP - delta) of every (query, key) pair, in the bias dtype, as a
     // full (B, H, Tq, Tk) tensor whose rows are padded to whole 64-key tiles (the caller sums broadcast dims)
     AttnTensor dbias;
+    // Tile classes of a bias shared by the heads (or words == null), read by the CLS variants of the kernels, and which
+    // workgroups this launch serves when the classes came with two launches (see cls_batch_dense): 0 all, 1 only batch
+    // elements whose bias is mostly ZERO / NEG tiles, 2 only the others.
+    BiasClasses cls;
+    int cls_take;
+    // dK/dV launches with classes: one byte per (batch, key block), written by the CLS launch (1: a key mask block, served
+    // there) and read by the ordinary launch behind it, which then need not look at the bias to know what is left for it
+    uint8_t* cls_served;
 };
 
 // block id -> (logical item, part, number of parts, part id)
@@ -159,17 +168,21 @@ template <int DPAD> struct DqSmem {
 // DBIAS: also write the bias gradient (a variant of its own: the kernels for head dims above 64 have no register to
 // spare, and a pointer that is only tested at run time already costs them spills in the main loop: config-4-sized
 // backward 0.31 -> 0.57 ms when it was a run-time option)
-template <typename T, int DPAD, int BIAS, bool DBIAS = false>
+// CLS: the bias comes with tile classes (attn_classes.h); the kernel is laid out like the one without bias, runs the
+// instructions of a tile without bias on ZERO tiles, leaves NEG tiles out and reads the bias of a MIXED tile in its step.
+template <typename T, int DPAD, int BIAS, bool DBIAS = false, bool CLS = false>
 __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32) ? 2 : 1) void attn_bwd_dq_kernel(const AttnBwdParams p) {
     constexpr bool HAS_BIAS = BIAS != BIAS_OFF;
     static_assert(!DBIAS || HAS_BIAS, "a bias gradient needs a bias");
+    static_assert(!CLS || (HAS_BIAS && !DBIAS && DPAD <= 64), "tile classes: head dims up to 64, with a bias, no bias gradient");
+    constexpr bool BIAS_AHEAD = HAS_BIAS && !CLS;  // bias registers fetched one tile ahead of use
     typedef typename BiasElem<T, BIAS>::type TB;
     typedef Mfma<T> MM;
     constexpr int BN = DqSmem<DPAD>::BN;
     constexpr int NKB = BN / 32;  // 32-key halves per tile
     // starting the dP accumulators from -delta takes 16 registers; the bias variants at two wavefronts per
     // SIMD have none to spare and subtract delta per element instead
-    constexpr bool DP_INIT = BIAS == BIAS_OFF || (DPAD > 64 && DqSmem<DPAD>::BN == 64);
+    constexpr bool DP_INIT = BIAS == BIAS_OFF || CLS || (DPAD > 64 && DqSmem<DPAD>::BN == 64);
     constexpr int ST = BwdTile<DPAD>::S;
     constexpr int TILE = DqSmem<DPAD>::TILE;
     constexpr int NC = DPAD / 16;
@@ -185,10 +198,15 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 31, g = lane >> 5;
     const BwdItem item = bwd_item(p);
-    const int bid = item.bid;
     int qb, bh;
-    row_block_of(bid, p.nblk, p.group_lg, p.causal != 0, qb, bh);  // causal: longest row blocks first
+    row_block_of(item.bid, p.nblk, p.group_lg, p.causal != 0, qb, bh);  // causal: longest row blocks first
     const int b = bh / p.H, h = bh - b * p.H;
+    if constexpr (HAS_BIAS && !DBIAS && DPAD <= 64) {
+        // classes came with two launches over the same grid: this one serves the batch elements of its kind
+        if (p.cls_take != 0) {
+            if (cls_batch_dense(p.cls, b, (p.Tk + CLS_KEYS - 1) / CLS_KEYS, lane) != (p.cls_take == 2)) return;
+        }
+    }
     const int q_row = qb * BWD_BM + wave * 32 + li;
     const bool q_valid = q_row < p.Tq;
     const int q_ld = q_valid ? q_row : p.Tq - 1;
@@ -262,7 +280,7 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
     }
     const bool fast_tiles = vec;  // rows made of whole 16-byte chunks
     // two staging register sets when the main loop fetches two tiles ahead (PF2), else one
-    constexpr bool PF2 = RGD_DQ_PREFETCH2 && DPAD <= 64 && !HAS_BIAS;
+    constexpr bool PF2 = RGD_DQ_PREFETCH2 && DPAD <= 64 && (!HAS_BIAS || CLS);
     u32x4 kst_[PF2 ? 2 : 1][LOADS], vst_[PF2 ? 2 : 1][LOADS];
     // FAST (compile time): the tile is known to be full and on the 16-byte path.  The main loop runs on FAST steps
     // only; with the element-wise loader of ragged tiles in the same loop the compiler waits for every outstanding
@@ -302,12 +320,6 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
             *reinterpret_cast<u32x4*>(vs_base + buf * TILE + soff[i]) = vst[i];
         }
     };
-    if (t_begin < t_end) {
-        issue_loads(t_begin, IntC<0>{}, IntC<0>{});
-        store_tiles(t_begin & 1, IntC<0>{});
-    }
-    __syncthreads();
-
     const int a_off = mfma_row_perm(li) * ST + g * 8;
     const int tr_off = ((lane & 15) >> 2) * ST + mfma_row_perm(((lane >> 4) & 1) * 16 + (lane & 3) * 4) + g * 16 * ST;
     const TB* bias_row = nullptr;
@@ -316,9 +328,15 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
     if constexpr (HAS_BIAS) {
         if constexpr (DBIAS)
             dbias_row = static_cast<TB*>(const_cast<void*>(p.dbias.ptr)) + b * p.dbias.sb + h * p.dbias.sh + (int64_t)q_ld * p.dbias.sn;
-        bias_row = static_cast<const TB*>(p.bias.ptr) + b * p.bias.sb + h * p.bias.sh + (int64_t)q_ld * p.bias.sn;
-        if (t_begin < t_end) bias_cur.load(bias_row, t_begin * BN, g, p.Tk, p.bias_vec && (t_begin + 1) * BN <= p.Tk);
+        if constexpr (!CLS) bias_row = static_cast<const TB*>(p.bias.ptr) + b * p.bias.sb + h * p.bias.sh + (int64_t)q_ld * p.bias.sn;
     }
+    const uint8_t* const cls_lds = smem_raw + DqSmem<DPAD>::BYTES;  // CLS: class of every key tile for the workgroup's 128 rows
+    if constexpr (CLS)
+        cls_tiles_to_lds(p.cls, b, qb * (BWD_BM / CLS_ROWS), BWD_BM / CLS_ROWS, (p.Tk + BN - 1) / BN, smem_raw + DqSmem<DPAD>::BYTES, tid);
+    int run_end = t_end;  // end of the run of tiles that is being worked on (all of them unless CLS)
+    // CLS: class of the tile of the next step, read from the table in LDS a step ahead (in a register of every lane; the
+    // step makes a scalar of it)
+    int cls_ahead = CLS_ZERO;
 
     // One key tile.  FAST: tiles j and j+1 are full tiles on the 16-byte path (and the bias, if any, is aligned).
     // AHEAD 0: the step fetches tile j+1 and stores it at its end.  AHEAD 1 / 2 (j even / odd): it fetches tile j+2
@@ -326,25 +344,32 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
     constexpr bool RECORD = attn_skip_masked(DPAD, BIAS) && !DBIAS;
     int live_first = 0x7fffffff, live_end = 0;
     // into the staging set of j's parity and stores tile j+1, fetched by the step before, from the other set.
-    auto tile_step = [&](const int j, auto FAST, auto AHEAD) __attribute__((always_inline)) {
+    // WBIAS: the tiles of the run have a bias (always, unless the tile classes say that they are ZERO).
+    auto tile_step = [&](const int j, auto FAST, auto AHEAD, auto WBIAS, const int tc) __attribute__((always_inline)) {
         constexpr bool F = decltype(FAST)::value != 0;
         constexpr int AH = decltype(AHEAD)::value;
         const int buf = j & 1;
         const int key0 = j * BN;
         const bool tail = !F && key0 + BN > p.Tk;
-        if (F || j + 1 < t_end) {
+        if (F || j + 1 < run_end) {
             if constexpr (AH == 0) issue_loads(j + 1, FAST, IntC<0>{});
             else issue_loads(j + 2, FAST, IntC<AH - 1>{});
-            if constexpr (HAS_BIAS)
+            if constexpr (BIAS_AHEAD)
                 bias_nxt.load(bias_row, key0 + BN, g, p.Tk, F || (p.bias_vec && key0 + 2 * BN <= p.Tk));
         }
+        // WB: the tile has a bias: the registers fetched a step ago, or (CLS: a run of MIXED tiles, which are few) read
+        // here, at the start of the tile's own step
+        auto body = [&](auto WB) __attribute__((always_inline)) {
+        constexpr bool WITH_BIAS = decltype(WB)::value != 0;
+        const BiasRuns<TB, NKB>& bias_use = bias_cur;
+
         const T* ks = ks_base + buf * TILE + a_off;
         const T* vs = vs_base + buf * TILE + a_off;
         // A tile whose bias is -inf for every (query, key) pair of this wavefront has P = 0 and dS = 0: the step is left
         // out.  RGD_DQ_SKIP_EARLY 1: tested before the first two products (the bias was requested a step earlier), 0: after.
         bool masked_tile = false;
 #if RGD_DQ_SKIP_EARLY
-        if constexpr (attn_skip_masked(DPAD, BIAS)) masked_tile = bias_cur.all_neg_inf(0, NKB);
+        if constexpr (attn_skip_masked(DPAD, BIAS)) masked_tile = bias_use.all_neg_inf(0, NKB);
 #endif
         if constexpr (RGD_DQ_SKIP_EARLY && RECORD) {
             if (!masked_tile) {
@@ -357,14 +382,41 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
         if (!masked_tile) {
 #pragma unroll
         for (int kb = 0; kb < NKB; ++kb) {
-#pragma unroll
-            for (int v = 0; v < 16; ++v) s[kb][v] = 0.f;
             if constexpr (DP_INIT) {
                 dp[kb] = dp_init;
             } else {
 #pragma unroll
                 for (int v = 0; v < 16; ++v) dp[kb][v] = 0.f;
             }
+        }
+#pragma unroll
+        for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) s[kb][v] = 0.f;
+        if constexpr (CLS) {
+            // A MIXED or COLUMN tile (few; tc is its class): the first product starts from the bias, in units of the raw
+            // scores, instead of from zero, and the tile goes on like every other tile.  The bias is read here, straight
+            // into the accumulators: no register is held for it while other tiles run, and the row address is formed here
+            // for the same reason.  COLUMN: every row of the tile is the first row of this wavefront's 32, which all its
+            // lanes read.
+            if (__builtin_expect(tc != CLS_ZERO, 0)) {
+            int row = tc == CLS_COLUMN ? min(qb * BWD_BM + wave * 32, p.Tq - 1) : q_ld;
+            asm volatile("" : "+v"(row));
+            const TB* here = static_cast<const TB*>(p.bias.ptr) + b * p.bias.sb + h * p.bias.sh + (int64_t)row * p.bias.sn;
+            const float per_score = kLog2e / p.scale_log2;
+#pragma unroll
+            for (int kb = 0; kb < NKB; ++kb) {
+                BiasRuns<TB, 1> half;
+                half.load(here, key0 + kb * 32, g, p.Tk, key0 + BN <= p.Tk);
+                float bias_h[16];
+                half.decode_run(0, bias_h);
+#pragma unroll
+                for (int v = 0; v < 16; ++v) s[kb][v] = bias_h[v] * per_score;
+            }
+            }
+        }
+#pragma unroll
+        for (int kb = 0; kb < NKB; ++kb) {
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
                 const u32x4 ka = *reinterpret_cast<const u32x4*>(ks + kb * 32 * ST + c * 16);
@@ -375,7 +427,7 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
         }
         }
 #if !RGD_DQ_SKIP_EARLY
-        if constexpr (attn_skip_masked(DPAD, BIAS)) masked_tile = bias_cur.all_neg_inf(0, NKB);
+        if constexpr (attn_skip_masked(DPAD, BIAS)) masked_tile = bias_use.all_neg_inf(0, NKB);
 #endif
         if constexpr (!RGD_DQ_SKIP_EARLY && RECORD) {
             if (!masked_tile) {
@@ -384,18 +436,20 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
             }
         }
         if (!masked_tile) {
-        float bias_v[NKB][16];
-        if constexpr (HAS_BIAS) bias_cur.decode(bias_v);
         // t = logit - lse (log2 domain)
+        {
+            float bias_v[NKB][16];
+            if constexpr (WITH_BIAS && !CLS) bias_use.decode(bias_v);
 #pragma unroll
-        for (int kb = 0; kb < NKB; ++kb)
+            for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                if constexpr (HAS_BIAS)
-                    s[kb][v] = fmaf(s[kb][v], p.scale_log2, fmaf(bias_v[kb][v], kLog2e, neg_lse_l2));
-                else
-                    s[kb][v] = fmaf(s[kb][v], p.scale_log2, neg_lse_l2);
-            }
+                for (int v = 0; v < 16; ++v) {
+                    if constexpr (WITH_BIAS && !CLS)
+                        s[kb][v] = fmaf(s[kb][v], p.scale_log2, fmaf(bias_v[kb][v], kLog2e, neg_lse_l2));
+                    else
+                        s[kb][v] = fmaf(s[kb][v], p.scale_log2, neg_lse_l2);
+                }
+        }
         const bool diag = p.causal && (key0 + BN - 1 > qb * BWD_BM + wave * 32);
         if (tail || diag) {
 #pragma unroll
@@ -465,36 +519,75 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
                 }
             }
         }
-        if (F || j + 1 < t_end) {
+        };  // body
+        body(WBIAS);
+        if (F || j + 1 < run_end) {
             store_tiles(buf ^ 1, IntC<(AH == 0 ? 0 : 2 - AH)>{});
-            if constexpr (HAS_BIAS) bias_cur = bias_nxt;
+            if constexpr (BIAS_AHEAD) bias_cur = bias_nxt;
         }
         __syncthreads();
     };
-    {
+    // CLS: the class of the tile goes into the step as a scalar (read from LDS a step ahead)
+    auto step = [&](const int j, auto FAST, auto AHEAD, auto WBIAS) __attribute__((always_inline)) {
+        if constexpr (CLS) {
+            const int tc = __builtin_amdgcn_readfirstlane(cls_ahead);
+            cls_ahead = cls_lds[min(j + 1, CLS_LDS_BYTES - 1)];
+            tile_step(j, FAST, AHEAD, IntC<0>{}, tc);
+        } else {
+            tile_step(j, FAST, AHEAD, WBIAS, 0);
+        }
+    };
+    // The tiles [rb, re), one after the other: the first tile is loaded and stored to LDS here, every step then works a
+    // tile (or two) ahead.  A kernel without tile classes has one run, all its tiles.
+    auto run_tiles = [&](const int rb, const int re, auto WBIAS) __attribute__((always_inline)) {
+        run_end = re;
+        if constexpr (CLS) cls_ahead = cls_lds[rb];
+        if (rb < re) {
+            issue_loads(rb, IntC<0>{}, IntC<0>{});
+            store_tiles(rb & 1, IntC<0>{});
+            if constexpr (BIAS_AHEAD) bias_cur.load(bias_row, rb * BN, g, p.Tk, p.bias_vec && (rb + 1) * BN <= p.Tk);
+        }
+        __syncthreads();
         // tiles below n_fast are full and take the 16-byte path; a FAST step also prefetches tile j+1
         const bool fast_ok = fast_tiles && (!HAS_BIAS || p.bias_vec);
-        const int n_fast = fast_ok ? min(t_end, p.Tk / BN) : t_begin;
-        int j = t_begin;
+        const int n_fast = fast_ok ? min(re, p.Tk / BN) : rb;
+        int j = rb;
         if constexpr (PF2) {
             if (n_fast - j >= 4) {
                 // tile j is in LDS; tile j+1 goes into flight here, each step then fetches two tiles ahead
                 if (j & 1) {
                     issue_loads(j + 1, IntC<1>{}, IntC<0>{});
-                    tile_step(j, IntC<1>{}, IntC<2>{});
+                    step(j, IntC<1>{}, IntC<2>{}, WBIAS);
                     ++j;
                 } else {
                     issue_loads(j + 1, IntC<1>{}, IntC<1>{});
                 }
                 for (; j + 3 < n_fast; j += 2) {
-                    tile_step(j, IntC<1>{}, IntC<1>{});
-                    tile_step(j + 1, IntC<1>{}, IntC<2>{});
+                    step(j, IntC<1>{}, IntC<1>{}, WBIAS);
+                    step(j + 1, IntC<1>{}, IntC<2>{}, WBIAS);
                 }
                 // tile j is in LDS and tile j+1 in flight; the steps below fetch it again
             }
         }
-        for (; j + 1 < n_fast; ++j) tile_step(j, IntC<1>{}, IntC<0>{});
-        for (; j < t_end; ++j) tile_step(j, IntC<0>{}, IntC<0>{});
+        for (; j + 1 < n_fast; ++j) step(j, IntC<1>{}, IntC<0>{}, WBIAS);
+        for (; j < re; ++j) step(j, IntC<0>{}, IntC<0>{}, WBIAS);
+    };
+    if constexpr (CLS) {
+        // Runs of tiles that are not NEG go through the loop (the loop of the kernel without bias, plus the addition of the
+        // bias on MIXED tiles); NEG runs (P = 0 and dS = 0) are left out, K/V loads and all.
+        int j = t_begin;
+        while (j < t_end) {
+            if (cls_lds_at(cls_lds, j) == CLS_NEG) {
+                ++j;
+                continue;
+            }
+            int e = j + 1;
+            while (e < t_end && cls_lds_at(cls_lds, e) != CLS_NEG) ++e;
+            run_tiles(j, e, IntC<0>{});
+            j = e;
+        }
+    } else {
+        run_tiles(t_begin, t_end, IntC<(HAS_BIAS ? 1 : 0)>{});
     }
 
     if constexpr (RECORD) {
@@ -619,12 +712,19 @@ template <typename TB> struct BiasColumn {
     __device__ __forceinline__ Bits bits(int v) const { return __builtin_bit_cast(Bits, raw[v]); }
 };
 
-template <typename T, int DPAD, int BIAS, bool FUSED = false>
-__global__ __launch_bounds__(BWD_THREADS, dkv_occupancy(DPAD, BIAS, FUSED)) void attn_bwd_dkv_kernel(const AttnBwdParams p) {
+// CLS: the bias comes with tile classes (attn_classes.h).  The kernel is the one without bias (same loop, two 32-row
+// sub-tiles per step); it serves the key blocks that a padding mask leaves as "key mask" blocks (cls_key_mask_block): their
+// hidden keys are treated like keys that do not exist.  Every other key block leaves at once and runs in the ordinary biased
+// kernel, which is launched over the same grid behind this one (cls_take == 2) and leaves the key mask blocks alone.
+template <typename T, int DPAD, int BIAS, bool FUSED = false, bool CLS = false>
+__global__ __launch_bounds__(BWD_THREADS, dkv_occupancy(DPAD, CLS ? BIAS_OFF : BIAS, FUSED)) void attn_bwd_dkv_kernel(const AttnBwdParams p) {
     constexpr bool HAS_BIAS = BIAS != BIAS_OFF;
+    static_assert(!CLS || (HAS_BIAS && !FUSED && DPAD <= 64), "tile classes: head dims up to 64, with a bias, two-kernel form");
+    constexpr bool BIAS_AHEAD = HAS_BIAS && !CLS;  // bias registers fetched one step ahead of use
     typedef typename BiasElem<T, BIAS>::type TB;
+    typedef TB TB_;
     typedef Mfma<T> MM;
-    constexpr int NSUB = dkv_nsub(DPAD, BIAS, FUSED);
+    constexpr int NSUB = dkv_nsub(DPAD, CLS ? BIAS_OFF : BIAS, FUSED);
     typedef DkvSmem<DPAD, NSUB, FUSED> SM;
     static_assert(!FUSED || DPAD <= 64, "the one-pass form keeps K^T in registers: head dims up to 64");
     constexpr int DS_ST = SM::DS_STRIDE;
@@ -646,13 +746,34 @@ __global__ __launch_bounds__(BWD_THREADS, dkv_occupancy(DPAD, BIAS, FUSED)) void
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 31, g = lane >> 5;
     const BwdItem item = bwd_item(p);
-    const int bid = item.bid;
     int kblk, bh;
-    dkv_block_of(bid, p, kblk, bh);
+    dkv_block_of(item.bid, p, kblk, bh);
     const int b = bh / p.H, h = bh - b * p.H;
     const int key = kblk * BWD_BM + wave * 32 + li;  // this lane's key
-    const bool k_valid = key < p.Tk;
+    bool k_valid = key < p.Tk;
     const int k_ld = k_valid ? key : p.Tk - 1;
+    bool no_key_hidden = true;    // CLS: no key of the workgroup is hidden by the bias
+    bool all_keys_hidden = false;  // CLS: every one is (a fully padded key block): dK = dV = 0 without a single step
+    if constexpr (HAS_BIAS && !FUSED && DPAD <= 64) {
+        // classes came with two launches over the same grid: key mask blocks run here when CLS, all others when not
+        if (p.cls_take != 0) {
+            uint8_t* served = p.cls_served + (int64_t)b * p.nblk + kblk;
+            if constexpr (CLS) {
+                const TB_* key_col = static_cast<const TB_*>(p.bias.ptr) + b * p.bias.sb + h * p.bias.sh + k_ld;
+                bool hidden, any_hidden, all_hidden;
+                const bool pure = cls_key_mask_block<TB_>(p.cls, key_col, p.bias.sn, b, kblk * (BWD_BM / CLS_KEYS),
+                                                          min((p.Tq + CLS_ROWS - 1) / CLS_ROWS, p.cls.nrow32), p.Tq, lane, tid,
+                                                          reinterpret_cast<int*>(smem_raw), hidden, any_hidden, all_hidden);
+                if (tid == 0) *served = pure ? 1 : 0;  // every head of the batch element writes the same value
+                if (!pure) return;
+                k_valid = k_valid && !hidden;
+                no_key_hidden = !any_hidden;
+                all_keys_hidden = all_hidden;
+            } else {
+                if (*served != 0) return;
+            }
+        }
+    }
     const bool vec = p.vec != 0;
 
     const T* kp = static_cast<const T*>(p.k.ptr) + b * p.k.sb + h * p.k.sh + (int64_t)k_ld * p.k.sn;
@@ -728,6 +849,7 @@ __global__ __launch_bounds__(BWD_THREADS, dkv_occupancy(DPAD, BIAS, FUSED)) void
     const int tile_first = p.causal ? min(ntiles_all, (kblk * BWD_BM) / BQ) : 0;
     int tile_begin = tile_first + (int)((int64_t)(ntiles_all - tile_first) * item.part / item.nparts);
     int ntiles = tile_first + (int)((int64_t)(ntiles_all - tile_first) * (item.part + 1) / item.nparts);
+    if (all_keys_hidden) ntiles = tile_begin;
 
     // Leading query tiles whose bias is -inf for every (query, key) pair of the workgroup give P = 0 and add nothing to dK
     // and dV (a block-causal bias: all queries before the key block).  They are found here, before anything else is
@@ -879,12 +1001,6 @@ __global__ __launch_bounds__(BWD_THREADS, dkv_occupancy(DPAD, BIAS, FUSED)) void
             st[BQ + tid] = row_st ? -delta_st : 0.f;
         }
     };
-    if (tile_begin < ntiles) {
-        issue_loads(tile_begin, IntC<0>{});
-        store_tiles(tile_begin & 1);
-    }
-    __syncthreads();
-
     const int a_off = mfma_row_perm(li) * ST + g * 8;
     const int tr_off = ((lane & 15) >> 2) * ST + mfma_row_perm(((lane >> 4) & 1) * 16 + (lane & 3) * 4) + g * 16 * ST;
 
@@ -904,8 +1020,8 @@ __global__ __launch_bounds__(BWD_THREADS, dkv_occupancy(DPAD, BIAS, FUSED)) void
     if constexpr (HAS_BIAS) {
         bias_base = static_cast<const TB*>(p.bias.ptr) + b * p.bias.sb + h * p.bias.sh;
         bias_lane_off = (uint32_t)k_ld + (uint32_t)(g * 16) * (uint32_t)p.bias.sn;
-        if (tile_begin < ntiles) bias_load(bias_cur, tile_begin, IntC<0>{});
     }
+    int run_end = ntiles;  // end of the run of steps that is being worked on
 
     // One tile of BQ query rows.  FAST: tile j+1 is a full tile on the 16-byte path.
     // NOMASK: every key of the workgroup exists and the launch is not causal, so no logit is masked (and the step
@@ -913,26 +1029,31 @@ __global__ __launch_bounds__(BWD_THREADS, dkv_occupancy(DPAD, BIAS, FUSED)) void
     // PING 0 / 1: one half of a pair of steps that swap the roles of the two bias register sets (0 uses bias_cur and
     // fills bias_nxt, 1 the other way round), so no step copies 16 registers per sub-tile; 2: a single step that
     // uses bias_cur and copies bias_nxt into it at its end.
-    auto tile_step = [&](const int j, auto FAST, auto NOMASK, auto PING) __attribute__((always_inline)) {
+    // WBIAS: the steps of the run have a bias (always, unless the tile classes say that they are ZERO).
+    auto tile_step = [&](const int j, auto FAST, auto NOMASK, auto PING, auto WBIAS) __attribute__((always_inline)) {
         constexpr bool F = decltype(FAST)::value != 0;
         constexpr bool NM = decltype(NOMASK)::value != 0;
         constexpr int PP = decltype(PING)::value;
-        BiasColumn<TB>(&b_use)[NSUB] = pick_ref<PP == 1>(bias_cur, bias_nxt);
         BiasColumn<TB>(&b_fill)[NSUB] = pick_ref<PP == 1>(bias_nxt, bias_cur);
         const int buf = j & 1;
-        if (F || j + 1 < ntiles) {
+        if (F || j + 1 < run_end) {
             issue_loads(j + 1, FAST);
-            if constexpr (HAS_BIAS) bias_load(b_fill, j + 1, FAST);
+            if constexpr (BIAS_AHEAD) bias_load(b_fill, j + 1, FAST);
         }
         dq_phase(j - 1);  // one-pass form: dQ of the previous tile, beside this tile's first products
         const T* qs = reinterpret_cast<const T*>(smem_raw + buf * BUFB);
         const T* dos = qs + TILE;
         const float* st = reinterpret_cast<const float*>(smem_raw + buf * BUFB + 2 * TILE * 2);
+        // The sub-tiles [U0, U1) of the step.  WB: they have a bias: the registers fetched a step ago, or (CLS) read here.
+        auto body = [&](auto WB, auto UB, auto UE) __attribute__((always_inline)) {
+        constexpr bool WITH_BIAS = decltype(WB)::value != 0;
+        constexpr int U0 = decltype(UB)::value, U1 = decltype(UE)::value;
+        BiasColumn<TB>(&b_use)[NSUB] = pick_ref<PP == 1>(bias_cur, bias_nxt);
 
         // the dP accumulators start from -delta of their query rows, so that product comes out as dP - delta
         f32x16 s[NSUB], dp[NSUB];
 #pragma unroll
-        for (int u = 0; u < NSUB; ++u)
+        for (int u = U0; u < U1; ++u)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const f32x4 c = *reinterpret_cast<const f32x4*>(st + BQ + u * 32 + g * 16 + 4 * i);
@@ -952,7 +1073,7 @@ __global__ __launch_bounds__(BWD_THREADS, dkv_occupancy(DPAD, BIAS, FUSED)) void
             u32x4 qa[2][NSUB], da[2][NSUB];
             auto read_step = [&](int c) __attribute__((always_inline)) {
 #pragma unroll
-                for (int u = 0; u < NSUB; ++u) {
+                for (int u = U0; u < U1; ++u) {
                     qa[c & 1][u] = *reinterpret_cast<const u32x4*>(qs + u * 32 * ST + a_off + c * 16);
                     da[c & 1][u] = *reinterpret_cast<const u32x4*>(dos + u * 32 * ST + a_off + c * 16);
                 }
@@ -963,7 +1084,7 @@ __global__ __launch_bounds__(BWD_THREADS, dkv_occupancy(DPAD, BIAS, FUSED)) void
                 if (c + 1 < NC) read_step(c + 1);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int u = 0; u < NSUB; ++u) {
+                for (int u = U0; u < U1; ++u) {
                     s[u] = MM::run(as_v8<T>(qa[c & 1][u]), kreg[c], s[u]);
                     dp[u] = MM::run(as_v8<T>(da[c & 1][u]), vreg[c], dp[u]);
                 }
@@ -973,7 +1094,7 @@ __global__ __launch_bounds__(BWD_THREADS, dkv_occupancy(DPAD, BIAS, FUSED)) void
 #pragma unroll
             for (int c = 0; c < NC; ++c)
 #pragma unroll
-                for (int u = 0; u < NSUB; ++u) {
+                for (int u = U0; u < U1; ++u) {
                     const u32x4 qa = *reinterpret_cast<const u32x4*>(qs + u * 32 * ST + a_off + c * 16);
                     s[u] = MM::run(as_v8<T>(qa), kreg[c], s[u]);
                     const u32x4 da = *reinterpret_cast<const u32x4*>(dos + u * 32 * ST + a_off + c * 16);
@@ -987,17 +1108,17 @@ __global__ __launch_bounds__(BWD_THREADS, dkv_occupancy(DPAD, BIAS, FUSED)) void
         if constexpr (attn_skip_masked(DPAD, BIAS)) {
             bool first = true;
 #pragma unroll
-            for (int u = 0; u < NSUB; ++u) first = first && b_use[u].first_is_neg_inf();
+            for (int u = U0; u < U1; ++u) first = first && b_use[u].first_is_neg_inf();
             if (__builtin_amdgcn_ballot_w64(!first) == 0) {
                 bool all = true;
 #pragma unroll
-                for (int u = 0; u < NSUB; ++u) all = all && b_use[u].lane_all_neg_inf();
+                for (int u = U0; u < U1; ++u) all = all && b_use[u].lane_all_neg_inf();
                 masked_step = __builtin_amdgcn_ballot_w64(!all) == 0;
             }
         }
         if (!masked_step) {
 #pragma unroll
-        for (int u = 0; u < NSUB; ++u) {
+        for (int u = U0; u < U1; ++u) {
             const int q0 = j * BQ + u * 32;
             // t = logit - lse (log2 domain)
             float nlse[16];
@@ -1007,7 +1128,7 @@ __global__ __launch_bounds__(BWD_THREADS, dkv_occupancy(DPAD, BIAS, FUSED)) void
 #pragma unroll
                 for (int e = 0; e < 4; ++e) nlse[4 * i + e] = a[e];
             }
-            if constexpr (HAS_BIAS) {
+            if constexpr (WITH_BIAS) {
                 float bias_r[16];
                 b_use[u].decode(bias_r);
 #pragma unroll
@@ -1089,32 +1210,44 @@ __global__ __launch_bounds__(BWD_THREADS, dkv_occupancy(DPAD, BIAS, FUSED)) void
             }
         }
         }  // !masked_step
-        if (F || j + 1 < ntiles) {
+        };  // body
+        body(WBIAS, IntC<0>{}, IntC<NSUB>{});
+        if (F || j + 1 < run_end) {
             store_tiles(buf ^ 1);
-            if constexpr (HAS_BIAS && PP == 2) {
+            if constexpr (BIAS_AHEAD && PP == 2) {
 #pragma unroll
                 for (int u = 0; u < NSUB; ++u) bias_cur[u] = bias_nxt[u];
             }
         }
         __syncthreads();
     };
-    {
+    // The steps [rb, re), one after the other: the first tile is loaded and stored to LDS here, every step then fetches
+    // the tile of the next.  A kernel without tile classes has one run, all its steps.
+    auto run_steps = [&](const int rb, const int re, auto WBIAS) __attribute__((always_inline)) {
+        run_end = re;
+        if (rb < re) {
+            issue_loads(rb, IntC<0>{});
+            store_tiles(rb & 1);
+            if constexpr (BIAS_AHEAD) bias_load(bias_cur, rb, IntC<0>{});
+        }
+        __syncthreads();
         // tiles below n_fast have all their query rows and take the 16-byte path; a FAST step prefetches tile j+1
-        const int n_fast = fast_tiles ? min(ntiles, p.Tq / BQ) : tile_begin;
-        int j = tile_begin;
-        if (!p.causal && (kblk + 1) * BWD_BM <= p.Tk) {
-            if constexpr (HAS_BIAS) {
+        const int n_fast = fast_tiles ? min(re, p.Tq / BQ) : rb;
+        int j = rb;
+        if (!p.causal && (kblk + 1) * BWD_BM <= p.Tk && no_key_hidden) {
+            if constexpr (BIAS_AHEAD) {
                 for (; j + 2 < n_fast; j += 2) {
-                    tile_step(j, IntC<1>{}, IntC<1>{}, IntC<0>{});
-                    tile_step(j + 1, IntC<1>{}, IntC<1>{}, IntC<1>{});
+                    tile_step(j, IntC<1>{}, IntC<1>{}, IntC<0>{}, WBIAS);
+                    tile_step(j + 1, IntC<1>{}, IntC<1>{}, IntC<1>{}, WBIAS);
                 }
             }
-            for (; j + 1 < n_fast; ++j) tile_step(j, IntC<1>{}, IntC<1>{}, IntC<2>{});
+            for (; j + 1 < n_fast; ++j) tile_step(j, IntC<1>{}, IntC<1>{}, IntC<2>{}, WBIAS);
         } else {
-            for (; j + 1 < n_fast; ++j) tile_step(j, IntC<1>{}, IntC<0>{}, IntC<2>{});
+            for (; j + 1 < n_fast; ++j) tile_step(j, IntC<1>{}, IntC<0>{}, IntC<2>{}, WBIAS);
         }
-        for (; j < ntiles; ++j) tile_step(j, IntC<0>{}, IntC<0>{}, IntC<2>{});
-    }
+        for (; j < re; ++j) tile_step(j, IntC<0>{}, IntC<0>{}, IntC<2>{}, WBIAS);
+    };
+    run_steps(tile_begin, ntiles, IntC<(BIAS_AHEAD ? 1 : 0)>{});
     if constexpr (FUSED) {
         if (tile_begin < ntiles) dq_phase(ntiles - 1);  // the last tile's dS is complete: the loop ended on a barrier
     }
@@ -1128,7 +1261,7 @@ __global__ __launch_bounds__(BWD_THREADS, dkv_occupancy(DPAD, BIAS, FUSED)) void
         }
         return;
     }
-    if (k_valid) {
+    if (key < p.Tk) {  // (a key hidden by the bias exists and gets its zeros)
         T* dkp = static_cast<T*>(const_cast<void*>(p.dk.ptr)) + b * p.dk.sb + h * p.dk.sh + (int64_t)key * p.dk.sn;
         T* dvp = static_cast<T*>(const_cast<void*>(p.dv.ptr)) + b * p.dv.sb + h * p.dv.sh + (int64_t)key * p.dv.sn;
 #pragma unroll

@@ -41,7 +41,16 @@
 #define RGD_FWD_LAZY_MAX 1
 #endif
 
+// the variant that reads tile classes (CLS): wavefronts per SIMD, and whether it fetches K/V two tiles ahead
+#ifndef RGD_CLS_FWD_OCC
+#define RGD_CLS_FWD_OCC 3
+#endif
+#ifndef RGD_CLS_FWD_PF2
+#define RGD_CLS_FWD_PF2 0
+#endif
+
 #include "attn_common.h"
+#include "attn_classes.h"
 
 constexpr int ATTN_BM = 128;  // query rows per workgroup
 constexpr int ATTN_BN = 64;   // keys per tile
@@ -63,6 +72,11 @@ struct AttnFwdParams {
     int trim;      // look for trailing all -inf bias tiles first (see bias_trim_end)
     float* part_o;   // (parts, 128, DPAD) fp32 accumulators, relative to the part's reference exponent
     float* part_ml;  // (parts, 128, 2): reference exponent (log2 domain), sum of probabilities
+    // Tile classes of a bias shared by the heads (or words == null), read by the CLS variant of the kernel.
+    // cls_take: which workgroups this launch serves when the classes came with two launches (see cls_batch_dense):
+    // 0 all, 1 only batch elements whose bias is mostly ZERO / NEG tiles, 2 only the others.
+    BiasClasses cls;
+    int cls_take;
 };
 
 template <int DPAD> struct AttnFwdSmem {
@@ -71,9 +85,14 @@ template <int DPAD> struct AttnFwdSmem {
     static constexpr size_t BYTES = 2 * 2 * TILE * 2;  // K and V, double buffered
 };
 
-template <typename T, int DPAD, int BIAS>
-__global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 : 2) void attn_fwd_kernel(const AttnFwdParams p) {
+// CLS: the bias comes with tile classes (attn_classes.h).  The kernel is then laid out like the one without bias (no
+// bias registers carried from tile to tile, three wavefronts per SIMD): ZERO tiles run the instructions of a tile without
+// bias, NEG tiles are left out, and a MIXED tile reads its bias at the start of its own step.
+template <typename T, int DPAD, int BIAS, bool CLS = false>
+__global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 && BIAS == BIAS_OFF) ? 3 : 2)) void attn_fwd_kernel(const AttnFwdParams p) {
     constexpr bool HAS_BIAS = BIAS != BIAS_OFF;
+    static_assert(!CLS || (HAS_BIAS && DPAD <= 64), "tile classes: head dims up to 64, with a bias");
+    constexpr bool BIAS_AHEAD = HAS_BIAS && !CLS;  // bias registers fetched one tile ahead of use
     typedef typename BiasElem<T, BIAS>::type TB;
     typedef Mfma<T> MM;
     typedef AttnFwdSmem<DPAD> SM;
@@ -112,6 +131,12 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
     row_block_of(bid, p.nqb, p.group_lg, p.causal != 0, qb, bh);
     const int b = bh / p.H;
     const int h = bh - b * p.H;
+    if constexpr (HAS_BIAS && DPAD <= 64) {
+        // classes came with two launches over the same grid: this one serves the batch elements of its kind
+        if (p.cls_take != 0) {
+            if (cls_batch_dense(p.cls, b, (p.Tk + ATTN_BN - 1) / ATTN_BN, lane) != (p.cls_take == 2)) return;
+        }
+    }
 
     const int q_row = qb * ATTN_BM + wave * 32 + li;  // this lane's query row
     const bool q_valid = q_row < p.Tq;
@@ -182,7 +207,7 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
     // rows made of whole 16-byte chunks: straight-line loads, no masking except in the last tile
     const bool fast_tiles = vec && p.D % 8 == 0;
     // two staging register sets when the main loop fetches two tiles ahead (PF2), else one
-    constexpr bool PF2 = RGD_FWD_PREFETCH2 && DPAD <= 64 && (!HAS_BIAS || RGD_FWD_PREFETCH2_BIAS);
+    constexpr bool PF2 = RGD_FWD_PREFETCH2 && DPAD <= 64 && (!HAS_BIAS || RGD_FWD_PREFETCH2_BIAS) && (!CLS || RGD_CLS_FWD_PF2);
     u32x4 kst_[PF2 ? 2 : 1][LOADS], vst_[PF2 ? 2 : 1][LOADS];
     // FAST (compile time): the caller knows the tile is full and the 16-byte path applies, so the loads are
     // straight-line code.  The main loop below runs on FAST steps only: with the element-wise loader of ragged
@@ -231,12 +256,6 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
         }
     };
 
-    if (t_begin < t_end) {
-        issue_loads(t_begin, IntC<0>{}, IntC<0>{});
-        store_tiles(t_begin & 1, IntC<0>{});
-    }
-    __syncthreads();
-
     // per-lane LDS offsets (elements) of the operand reads; everything else is a compile-time offset
     const int a_off = mfma_row_perm(li) * ST + g * 8;  // K rows as A operand
     const int tr_off = ((lane & 15) >> 2) * ST + mfma_row_perm(((lane >> 4) & 1) * 16 + (lane & 3) * 4) +
@@ -245,32 +264,39 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
     // bias of this lane's query row, fetched one tile ahead of its use
     const TB* bias_row = nullptr;
     BiasRuns<TB> bias_cur, bias_nxt;
-    if constexpr (HAS_BIAS) {
+    const uint8_t* const cls_lds = smem_raw + SM::BYTES;  // CLS: class of every key tile for the workgroup's 128 rows
+    if constexpr (HAS_BIAS && !CLS)
         bias_row = static_cast<const TB*>(p.bias.ptr) + b * p.bias.sb + h * p.bias.sh + (int64_t)q_ld * p.bias.sn;
-        if (t_begin < t_end)
-            bias_cur.load(bias_row, t_begin * ATTN_BN, g, p.Tk, p.bias_vec && (t_begin + 1) * ATTN_BN <= p.Tk);
-    }
+    if constexpr (CLS)
+        cls_tiles_to_lds(p.cls, b, qb * (ATTN_BM / CLS_ROWS), ATTN_BM / CLS_ROWS, (p.Tk + ATTN_BN - 1) / ATTN_BN, smem_raw + SM::BYTES, tid);
+    int run_end = t_end;  // end of the run of tiles that is being worked on (all of them unless CLS)
+    // CLS: class of the tile of the next step, read from the table in LDS a step ahead (in a register of every lane; the
+    // step makes a scalar of it)
+    int cls_ahead = CLS_ZERO;
 
     // One key tile.  FAST: tiles j and j+1 are full tiles on the 16-byte path (and the bias, if any, is aligned).
     // AHEAD 0: the step fetches tile j+1 and stores it at its end.  AHEAD 1 / 2 (j even / odd): it fetches tile j+2
     // into the staging set of j's parity and stores tile j+1, fetched by the step before, from the other set: the
     // store no longer waits for loads issued a step ago at most.
-    auto tile_step = [&](const int j, auto FAST, auto AHEAD) __attribute__((always_inline)) {
+    // WBIAS: the tiles of the run have a bias (always, unless the tile classes say that they are ZERO).
+    auto tile_step = [&](const int j, auto FAST, auto AHEAD, auto WBIAS, const int tc) __attribute__((always_inline)) {
         constexpr bool F = decltype(FAST)::value != 0;
         constexpr int AH = decltype(AHEAD)::value;
         const int buf = j & 1;
         const int key0 = j * ATTN_BN;
         const bool tail = !F && key0 + ATTN_BN > p.Tk;
-        if (F || j + 1 < t_end) {
+        if (F || j + 1 < run_end) {
             if constexpr (AH == 0) issue_loads(j + 1, FAST, IntC<0>{});
             else issue_loads(j + 2, FAST, IntC<AH - 1>{});
-            if constexpr (HAS_BIAS)
+            if constexpr (BIAS_AHEAD)
                 bias_nxt.load(bias_row, key0 + ATTN_BN, g, p.Tk, F || (p.bias_vec && key0 + 2 * ATTN_BN <= p.Tk));
         }
         if constexpr (!SPLIT_HALVES) {
-            // d <= 64: both 32-key halves of the tile go through the softmax together
-            // A tile whose bias is -inf for every (query, key) pair of this wavefront adds nothing (p = 0 exactly):
-            // its products and its softmax are left out.
+            // d <= 64: both 32-key halves of the tile go through the softmax together.
+            // WB: the tile has a bias: the registers fetched a step ago, or (CLS, a MIXED tile) read here.
+            auto body = [&](auto WB) __attribute__((always_inline)) {
+            constexpr bool WITH_BIAS = decltype(WB)::value != 0;
+            const BiasRuns<TB>& bias_use = bias_cur;
 
             // ---- S^T = K . Q^T ----
             const T* ks = ks_base + buf * TILE + a_off;
@@ -279,6 +305,29 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) s[kb][v] = 0.f;
+            if constexpr (CLS) {
+                // A MIXED or COLUMN tile (few; tc is its class): the product starts from the bias, in units of the raw
+                // scores, instead of from zero, and the tile goes on like every other tile.  The bias is read here, straight
+                // into the accumulators: no register is held for it while other tiles run, and the row address is formed
+                // here for the same reason.  COLUMN: every row of the tile is the first row of this wavefront's 32, which
+                // all its lanes read.  (A copy of the whole step for these tiles, which would leave the step of the other
+                // tiles exactly that of the kernel without bias, costs that step registers it does not have: spills.)
+                if (__builtin_expect(tc != CLS_ZERO, 0)) {
+                int row = tc == CLS_COLUMN ? min(qb * ATTN_BM + wave * 32, p.Tq - 1) : q_ld;
+                asm volatile("" : "+v"(row));
+                const TB* here = static_cast<const TB*>(p.bias.ptr) + b * p.bias.sb + h * p.bias.sh + (int64_t)row * p.bias.sn;
+                const float per_score = kLog2e / p.scale_log2;
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb) {
+                    BiasRuns<TB, 1> half;
+                    half.load(here, key0 + kb * 32, g, p.Tk, key0 + ATTN_BN <= p.Tk);
+                    float bias_v[16];
+                    half.decode_run(0, bias_v);
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) s[kb][v] = bias_v[v] * per_score;
+                }
+                }
+            }
             // the two halves alternate, so consecutive matrix instructions never wait for each other's result
 #pragma unroll
             for (int c = 0; c < NC; ++c)
@@ -288,19 +337,13 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
                     s[kb] = MM::run(as_v8<T>(a), qreg[c], s[kb]);
                 }
 
-            // A tile whose bias is -inf for every (query, key) pair of this wavefront adds nothing (p = 0 exactly):
-            // its softmax and its second product are left out.  The test sits where the bias is first needed, after
-            // the first product has been issued, so the bias loads keep the time of that product to arrive.
-            bool masked_tile = false;
-            if constexpr (attn_skip_masked(DPAD, BIAS)) masked_tile = bias_cur.all_neg_inf(0, 2);
-            if (!masked_tile) {
             // ---- t = logit - m_ref (log2 domain) ----
             const float m_off = m_ref == -INFINITY ? 0.f : m_ref;
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb) {
-                if constexpr (HAS_BIAS) {
+                if constexpr (WITH_BIAS && !CLS) {
                     float bias_v[16];
-                    bias_cur.decode_run(kb, bias_v);
+                    bias_use.decode_run(kb, bias_v);
 #pragma unroll
                     for (int v = 0; v < 16; ++v) s[kb][v] = fmaf(s[kb][v], p.scale_log2, fmaf(bias_v[v], kLog2e, -m_off));
                 } else {
@@ -401,7 +444,8 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
                     oacc[d] = MM::run(as_v8<T>(a), pb, oacc[d]);
                 }
             }
-            }  // !masked_tile
+            };  // body
+            body(WBIAS);
         } else {
             // Each 32-key half of the tile is a complete softmax step of its own (S -> p -> PV), so only 16
             // logits are live at a time; the register budget buys wavefronts per SIMD, and those hide the
@@ -500,36 +544,73 @@ __global__ __launch_bounds__(ATTN_THREADS, (DPAD <= 64 && BIAS == BIAS_OFF) ? 3 
             }
         }
 
-        if (F || j + 1 < t_end) {
+        if (F || j + 1 < run_end) {
             store_tiles(buf ^ 1, IntC<(AH == 0 ? 0 : 2 - AH)>{});
-            if constexpr (HAS_BIAS) bias_cur = bias_nxt;
+            if constexpr (BIAS_AHEAD) bias_cur = bias_nxt;
         }
         __syncthreads();
     };
-    {
+    // CLS: the class of the tile goes into the step as a scalar (read from LDS a step ahead)
+    auto step = [&](const int j, auto FAST, auto AHEAD, auto WBIAS) __attribute__((always_inline)) {
+        if constexpr (CLS) {
+            const int tc = __builtin_amdgcn_readfirstlane(cls_ahead);
+            cls_ahead = cls_lds[min(j + 1, CLS_LDS_BYTES - 1)];
+            tile_step(j, FAST, AHEAD, IntC<0>{}, tc);
+        } else {
+            tile_step(j, FAST, AHEAD, WBIAS, 0);
+        }
+    };
+    // The tiles [rb, re), one after the other: the first tile is loaded and stored to LDS here, every step then works a
+    // tile (or two) ahead.  A kernel without tile classes has one run, all its tiles.
+    auto run_tiles = [&](const int rb, const int re, auto WBIAS) __attribute__((always_inline)) {
+        run_end = re;
+        if constexpr (CLS) cls_ahead = cls_lds[rb];
+        if (rb < re) {
+            issue_loads(rb, IntC<0>{}, IntC<0>{});
+            store_tiles(rb & 1, IntC<0>{});
+            if constexpr (BIAS_AHEAD) bias_cur.load(bias_row, rb * ATTN_BN, g, p.Tk, p.bias_vec && (rb + 1) * ATTN_BN <= p.Tk);
+        }
+        __syncthreads();
         // tiles below n_fast are full and take the 16-byte path; a FAST step also prefetches tile j+1
         const bool fast_ok = fast_tiles && (!HAS_BIAS || p.bias_vec);
-        const int n_fast = fast_ok ? min(t_end, p.Tk / ATTN_BN) : t_begin;
-        int j = t_begin;
+        const int n_fast = fast_ok ? min(re, p.Tk / ATTN_BN) : rb;
+        int j = rb;
         if constexpr (PF2) {
             if (n_fast - j >= 4) {
                 // tile j is in LDS; tile j+1 goes into flight here, each step then fetches two tiles ahead
                 if (j & 1) {
                     issue_loads(j + 1, IntC<1>{}, IntC<0>{});
-                    tile_step(j, IntC<1>{}, IntC<2>{});
+                    step(j, IntC<1>{}, IntC<2>{}, WBIAS);
                     ++j;
                 } else {
                     issue_loads(j + 1, IntC<1>{}, IntC<1>{});
                 }
                 for (; j + 3 < n_fast; j += 2) {
-                    tile_step(j, IntC<1>{}, IntC<1>{});
-                    tile_step(j + 1, IntC<1>{}, IntC<2>{});
+                    step(j, IntC<1>{}, IntC<1>{}, WBIAS);
+                    step(j + 1, IntC<1>{}, IntC<2>{}, WBIAS);
                 }
                 // tile j is in LDS and tile j+1 in flight (set of its parity); the steps below fetch it again
             }
         }
-        for (; j + 1 < n_fast; ++j) tile_step(j, IntC<1>{}, IntC<0>{});
-        for (; j < t_end; ++j) tile_step(j, IntC<0>{}, IntC<0>{});
+        for (; j + 1 < n_fast; ++j) step(j, IntC<1>{}, IntC<0>{}, WBIAS);
+        for (; j < re; ++j) step(j, IntC<0>{}, IntC<0>{}, WBIAS);
+    };
+    if constexpr (CLS) {
+        // Runs of tiles that are not NEG go through the loop (the loop of the kernel without bias, plus the addition of the
+        // bias on MIXED tiles); NEG runs (every probability 0) are left out, K/V loads and all.
+        int j = t_begin;
+        while (j < t_end) {
+            if (cls_lds_at(cls_lds, j) == CLS_NEG) {
+                ++j;
+                continue;
+            }
+            int e = j + 1;
+            while (e < t_end && cls_lds_at(cls_lds, e) != CLS_NEG) ++e;
+            run_tiles(j, e, IntC<0>{});
+            j = e;
+        }
+    } else {
+        run_tiles(t_begin, t_end, IntC<(HAS_BIAS ? 1 : 0)>{});
     }
 
     const float l_tot = l_run + lane_xor32(l_run);

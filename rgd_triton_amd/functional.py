@@ -490,7 +490,22 @@ def _bias_args(bias, q, seqlen_q, seqlen_k, batch, nheads):
     return desc, kind, _hip.dtype_code(bias.dtype)
 
 
-def _flash_attn_forward(q, k, v, bias=None, causal=False, softmax_scale=None, kernel_cache=None):
+def _bias_classes(bias, bdesc, bkind, bdtype, dims):
+    """Tile classes of a bias matrix that the heads share (rgd_attn_bias_classify): one pass over the bias, made in the
+    forward and kept for the backward.  None when the library has no use for them (any other bias, head dims above 64)."""
+    if bias is None:
+        return None
+    lib = _hip.lib()
+    nbytes = lib.rgd_attn_bias_classes_bytes(*dims, bdesc, bkind, bdtype)
+    if nbytes == 0:
+        return None
+    classes = torch.empty(nbytes // 8, dtype=torch.int64, device=bias.device)
+    _hip.check(lib.rgd_attn_bias_classify(*dims, bdesc, bkind, bdtype, classes.data_ptr(), nbytes, _hip.stream_ptr(bias.device)),
+               "rgd_attn_bias_classify")
+    return classes
+
+
+def _flash_attn_forward(q, k, v, bias=None, causal=False, softmax_scale=None, kernel_cache=None, return_classes=False):
     batch, seqlen_q, nheads, d = q.shape
     _, seqlen_k, _, _ = k.shape
     if not _seen(kernel_cache, "fwd", _sig(q, k, v, bias) + (bool(causal),)):
@@ -509,10 +524,14 @@ def _flash_attn_forward(q, k, v, bias=None, causal=False, softmax_scale=None, ke
     lse = torch.empty((batch, nheads, seqlen_q_rounded), device=q.device, dtype=torch.float32)
     o = torch.empty_like(q)
     ws = _hip.workspace(q.device, lib.rgd_attn_fwd_workspace(batch, nheads, seqlen_q, seqlen_k, d))
+    classes = _bias_classes(bias, bdesc, bkind, bdtype, (batch, nheads, seqlen_q, seqlen_k, d))
     _hip.check(lib.rgd_attn_fwd(batch, nheads, seqlen_q, seqlen_k, d, t4(q, False), t4(k, False), t4(v, False),
                                 bdesc, bkind, bdtype, t4(o, False), ctypes.c_void_p(lse.data_ptr()),
                                 _hip.dtype_code(q.dtype), int(bool(causal)), float(softmax_scale),
+                                classes.data_ptr() if classes is not None else None,
                                 ctypes.c_void_p(ws.data_ptr()), ws.numel(), _hip.stream_ptr(q.device)), "rgd_attn_fwd")
+    if return_classes:
+        return o, lse, softmax_scale, classes
     return o, lse, softmax_scale
 
 
@@ -541,7 +560,7 @@ def _bwd_mode(d):
 
 
 def _flash_attn_backward(do, q, k, v, o, lse, dq, dk, dv, bias=None, causal=False, softmax_scale=None,
-                         kernel_cache=None, bias_grad=False):
+                         kernel_cache=None, bias_grad=False, bias_classes=None):
     """Returns None, or with bias_grad the gradient of `bias` in its own shape and dtype (beyond the reference, which
     refuses it, flash_attn_triton_cached.py:1107): the dQ kernel leaves dS of every (query, key) pair in a full
     (B, H, Tq, Tk) buffer and the dimensions the bias broadcasts are summed here in fp32."""
@@ -572,7 +591,8 @@ def _flash_attn_backward(do, q, k, v, o, lse, dq, dk, dv, bias=None, causal=Fals
     _hip.check(lib.rgd_attn_bwd(batch, nheads, seqlen_q, seqlen_k, d, t4(do, False), t4(q, False), t4(k, False),
                                 t4(v, False), t4(o, False), ctypes.c_void_p(lse.data_ptr()), bdesc, bkind, bdtype,
                                 t4(dq, False), t4(dk, False), t4(dv, False), ddesc, _hip.dtype_code(q.dtype),
-                                int(bool(causal)), float(softmax_scale), mode, ws.data_ptr(), nbytes,
+                                int(bool(causal)), float(softmax_scale), mode,
+                                bias_classes.data_ptr() if bias_classes is not None else None, ws.data_ptr(), nbytes,
                                 _hip.stream_ptr(q.device)), "rgd_attn_bwd")
     if not bias_grad:
         return None
@@ -592,8 +612,8 @@ class FlashAttnFunc(torch.autograd.Function):
         bias: optional, shape broadcastible to (batch, nheads, seqlen_q, seqlen_k).
         """
         q, k, v, bias = _lastdim_contig(q, k, v, bias)
-        o, lse, ctx.softmax_scale = _flash_attn_forward(q, k, v, bias=bias, causal=causal, softmax_scale=softmax_scale,
-                                                        kernel_cache=kernel_cache)
+        o, lse, ctx.softmax_scale, ctx.bias_classes = _flash_attn_forward(
+            q, k, v, bias=bias, causal=causal, softmax_scale=softmax_scale, kernel_cache=kernel_cache, return_classes=True)
         ctx.kernel_cache = kernel_cache
         ctx.save_for_backward(q, k, v, o, lse, bias)
         ctx.causal = causal
@@ -609,7 +629,7 @@ class FlashAttnFunc(torch.autograd.Function):
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
         dbias = _flash_attn_backward(do, q, k, v, o, lse, dq, dk, dv, bias=bias, causal=ctx.causal,
                                      softmax_scale=ctx.softmax_scale, kernel_cache=ctx.kernel_cache,
-                                     bias_grad=bias is not None and ctx.needs_input_grad[3])
+                                     bias_grad=bias is not None and ctx.needs_input_grad[3], bias_classes=ctx.bias_classes)
         return dq, dk, dv, dbias, None, None, None
 
 

@@ -22,7 +22,7 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), f"{name} declared in include/rgd_hip.h but not exported"
         assert name in _hip._SIGNATURES, f"{name} has no ctypes signature"
     assert sorted(_hip._SIGNATURES) == declared
-    assert lib.rgd_version() == 2000 and lib.rgd_version() // 1000 == _hip.ABI_MAJOR
+    assert lib.rgd_version() == 3000 and lib.rgd_version() // 1000 == _hip.ABI_MAJOR
     assert lib.rgd_attn_seqlen_q_rounded(1) == 64 and lib.rgd_attn_seqlen_q_rounded(128) == 128
     assert lib.rgd_attn_seqlen_q_rounded(129) == 192
     # delta (required part) plus room for the partial sums of split workgroups
@@ -50,7 +50,7 @@ def test_error_paths_return_codes_without_a_gpu():
     for pos in range(4):  # dout, q, k, v in turn
         args = [t4] * 5
         args[pos] = far
-        assert lib.rgd_attn_bwd(1, 1, 8, 8, 64, *args, 0x1000, None, 0, 0, t4, t4, t4, None, 1, 0, 0.125, 1, 0x1000, 1 << 20,
+        assert lib.rgd_attn_bwd(1, 1, 8, 8, 64, *args, 0x1000, None, 0, 0, t4, t4, t4, None, 1, 0, 0.125, 1, None, 0x1000, 1 << 20,
                                 None) == -2, pos
         assert b"token stride" in lib.rgd_last_error()
     assert lib.rgd_ln_qk_fwd(1, 1, 4, 4, 300, t4, t4, t4, t4, 0, 1e-6, None) == -1
@@ -58,20 +58,20 @@ def test_error_paths_return_codes_without_a_gpu():
     assert lib.rgd_rope_qk(1, 1, 4, 4, 160, t4, t4, t4, t4, 0x1000, 8, 32, 256, 32, 0, 4, 4, 0, 0, None) == -1
     assert b"head dimensions up to 128" in lib.rgd_last_error()
     assert lib.rgd_rope_qk(1, 1, 8, 8, 64, t4, t4, t4, t4, 0x1000, 8, 32, 256, 32, 0, 8, 8, 0, 0, None) == -1  # T < P
-    assert lib.rgd_attn_fwd(1, 1, 8, 8, 64, t4, t4, t4, None, 0, 0, t4, 0x1000, 0, 0, 0.125, None, 0, None) == -1
+    assert lib.rgd_attn_fwd(1, 1, 8, 8, 64, t4, t4, t4, None, 0, 0, t4, 0x1000, 0, 0, 0.125, None, None, 0, None) == -1
     assert b"Only support fp16 and bf16" in lib.rgd_last_error()
-    assert lib.rgd_attn_fwd(1, 1, 8, 8, 200, t4, t4, t4, None, 0, 0, t4, 0x1000, 1, 0, 0.125, None, 0, None) == -1
+    assert lib.rgd_attn_fwd(1, 1, 8, 8, 200, t4, t4, t4, None, 0, 0, t4, 0x1000, 1, 0, 0.125, None, None, 0, None) == -1
     assert b"head dimensions up to 128" in lib.rgd_last_error()
-    assert lib.rgd_attn_fwd(1, 1, 8, 8, 64, t4, t4, t4, t4, 2, 2, t4, 0x1000, 1, 0, 0.125, None, 0, None) == -1  # bias dtype
-    assert lib.rgd_attn_bwd(1, 1, 8, 8, 64, t4, t4, t4, t4, t4, 0x1000, None, 0, 0, t4, t4, t4, None, 1, 0, 0.125, 1, 0x1000, 16,
+    assert lib.rgd_attn_fwd(1, 1, 8, 8, 64, t4, t4, t4, t4, 2, 2, t4, 0x1000, 1, 0, 0.125, None, None, 0, None) == -1  # bias dtype
+    assert lib.rgd_attn_bwd(1, 1, 8, 8, 64, t4, t4, t4, t4, t4, 0x1000, None, 0, 0, t4, t4, t4, None, 1, 0, 0.125, 1, None, 0x1000, 16,
                             None) == -4
     # the one-pass form needs room for dq_accum behind delta, and exists for head dims up to 64
     assert lib.rgd_attn_bwd_workspace(1, 1, 8, 8, 64, 2) >= 64 * 4 + 64 * 64 * 4
-    assert lib.rgd_attn_bwd(1, 1, 8, 8, 64, t4, t4, t4, t4, t4, 0x1000, None, 0, 0, t4, t4, t4, None, 1, 0, 0.125, 2, 0x1000, 1024,
+    assert lib.rgd_attn_bwd(1, 1, 8, 8, 64, t4, t4, t4, t4, t4, 0x1000, None, 0, 0, t4, t4, t4, None, 1, 0, 0.125, 2, None, 0x1000, 1024,
                             None) == -4
-    assert lib.rgd_attn_bwd(1, 1, 8, 8, 128, t4, t4, t4, t4, t4, 0x1000, None, 0, 0, t4, t4, t4, None, 1, 0, 0.125, 2, 0x1000,
+    assert lib.rgd_attn_bwd(1, 1, 8, 8, 128, t4, t4, t4, t4, t4, 0x1000, None, 0, 0, t4, t4, t4, None, 1, 0, 0.125, 2, None, 0x1000,
                             1 << 20, None) == -2
-    assert lib.rgd_attn_bwd(1, 1, 8, 8, 64, t4, t4, t4, t4, t4, 0x1000, None, 0, 0, t4, t4, t4, None, 1, 0, 0.125, 7, 0x1000,
+    assert lib.rgd_attn_bwd(1, 1, 8, 8, 64, t4, t4, t4, t4, t4, 0x1000, None, 0, 0, t4, t4, t4, None, 1, 0, 0.125, 7, None, 0x1000,
                             1 << 20, None) == -1
     # zero-sized problems are a successful no-op
     assert lib.rgd_l2_fwd(0, 0, 8, t3, t3, 0, 1e-6, None) == 0

@@ -411,14 +411,14 @@ def test_flash_attn_bwd_key_ranges(d, Tq, Tk, pattern, bias_shape, dtype):
     lse = torch.empty(B, H, tqr, dtype=torch.float32, device="cuda")
     t = {n: _hip.t4(x, False) for n, x in dict(q=qg, k=kg, v=vg, do=dog, o=o).items()}
     assert lib.rgd_attn_fwd(B, H, Tq, Tk, d, t["q"], t["k"], t["v"], bdesc, kind, code, t["o"], lse.data_ptr(), code, 0, scale,
-                            None, 0, st) == 0, lib.rgd_last_error()
+                            None, None, 0, st) == 0, lib.rgd_last_error()
 
     def run(bws_bytes):
         dq, dk, dv = torch.empty_like(qg), torch.empty_like(kg), torch.empty_like(vg)
         bws = torch.empty(bws_bytes, dtype=torch.uint8, device="cuda")
         tt = {n: _hip.t4(x, False) for n, x in dict(dq=dq, dk=dk, dv=dv).items()}
         rc = lib.rgd_attn_bwd(B, H, Tq, Tk, d, t["do"], t["q"], t["k"], t["v"], t["o"], lse.data_ptr(), bdesc, kind, code,
-                              tt["dq"], tt["dk"], tt["dv"], None, code, 0, scale, 1, bws.data_ptr(), bws_bytes, st)
+                              tt["dq"], tt["dk"], tt["dv"], None, code, 0, scale, 1, None, bws.data_ptr(), bws_bytes, st)
         assert rc == 0, lib.rgd_last_error()
         torch.cuda.synchronize()
         return dq, dk, dv
@@ -707,10 +707,10 @@ def test_flash_attn_split_workgroups(B, H, T, d, with_bias, mode, dtype):
         bws = torch.empty(bws_bytes, dtype=torch.uint8, device="cuda")
         t = {n: _hip.t4(x, False) for n, x in dict(q=qg, k=kg, v=vg, do=dog, o=o, dq=dq, dk=dk, dv=dv).items()}
         rc = lib.rgd_attn_fwd(B, H, T, T, d, t["q"], t["k"], t["v"], bdesc, bk, bd, t["o"], lse.data_ptr(), code, 0, scale,
-                              fws.data_ptr() if fws_bytes else None, fws_bytes, st)
+                              None, fws.data_ptr() if fws_bytes else None, fws_bytes, st)
         assert rc == 0, lib.rgd_last_error()
         rc = lib.rgd_attn_bwd(B, H, T, T, d, t["do"], t["q"], t["k"], t["v"], t["o"], lse.data_ptr(), bdesc, bk, bd, t["dq"],
-                              t["dk"], t["dv"], None, code, 0, scale, mode, bws.data_ptr(), bws_bytes, st)
+                              t["dk"], t["dv"], None, code, 0, scale, mode, None, bws.data_ptr(), bws_bytes, st)
         assert rc == 0, lib.rgd_last_error()
         torch.cuda.synchronize()
         return o, lse, dq, dk, dv

@@ -67,11 +67,11 @@ class _Sequence:
         scale = 1.0 / math.sqrt(D)
         # attention consumes the LN+RoPE outputs of this same sequence
         rc |= lib.rgd_attn_fwd(B, H, T, T, D, t4(out["qo"]), t4(out["ko"]), t4(i["v"]), bdesc, hip.BIAS_MATRIX, code,
-                               t4(out["o"]), self.lse.data_ptr(), code, 0, scale, self.attn_fws.data_ptr(),
+                               t4(out["o"]), self.lse.data_ptr(), code, 0, scale, None, self.attn_fws.data_ptr(),
                                self.attn_fws.numel(), st)
         rc |= lib.rgd_attn_bwd(B, H, T, T, D, t4(i["g1"]), t4(out["qo"]), t4(out["ko"]), t4(i["v"]), t4(out["o"]),
                                self.lse.data_ptr(), bdesc, hip.BIAS_MATRIX, code, t4(out["dq"]), t4(out["dk"]),
-                               t4(out["dv"]), None, code, 0, scale, 1, self.attn_ws.data_ptr(), self.attn_ws.numel(), st)
+                               t4(out["dv"]), None, code, 0, scale, 1, None, self.attn_ws.data_ptr(), self.attn_ws.numel(), st)
         assert rc == 0, lib.rgd_last_error()
 
 
