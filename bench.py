@@ -296,7 +296,7 @@ def time_api(torch, fn, iters=30, warmup=5):
     return a.elapsed_time(b) / iters
 
 
-def attention_case(torch, name, B, T, H, D, dtype, bias_kind, iters=20, with_cpu=False):
+def attention_case(torch, name, B, T, H, D, dtype, bias_kind, iters=20, with_cpu=False, causal=False):
     """fwd+bwd through the C ABI with events around the forward and the backward call"""
     from rgd_triton_amd import _hip
 
@@ -347,12 +347,12 @@ def attention_case(torch, name, B, T, H, D, dtype, bias_kind, iters=20, with_cpu
     def fwd():
         if cls_bytes:
             assert lib.rgd_attn_bias_classify(B, H, T, T, D, bdesc, bk, bd, cls_ptr, cls_bytes, st) == 0, lib.rgd_last_error()
-        assert lib.rgd_attn_fwd(B, H, T, T, D, t["q"], t["k"], t["v"], bdesc, bk, bd, t["o"], lse.data_ptr(), code, 0,
+        assert lib.rgd_attn_fwd(B, H, T, T, D, t["q"], t["k"], t["v"], bdesc, bk, bd, t["o"], lse.data_ptr(), code, int(causal),
                                 scale, cls_ptr, fws.data_ptr(), fws.numel(), st) == 0, lib.rgd_last_error()
 
     def bwd():
         assert lib.rgd_attn_bwd(B, H, T, T, D, t["do"], t["q"], t["k"], t["v"], t["o"], lse.data_ptr(), bdesc, bk, bd,
-                                t["dq"], t["dk"], t["dv"], None, code, 0, scale, mode, cls_ptr, ws.data_ptr(), ws.numel(), st) == 0, \
+                                t["dq"], t["dk"], t["dv"], None, code, int(causal), scale, mode, cls_ptr, ws.data_ptr(), ws.numel(), st) == 0, \
             lib.rgd_last_error()
 
     # forward and backward alternate as in a training step; the clocks are brought to their steady state first
@@ -373,12 +373,11 @@ def attention_case(torch, name, B, T, H, D, dtype, bias_kind, iters=20, with_cpu
     torch.cuda.synchronize()
     f_ms = statistics.mean(e[0].elapsed_time(e[1]) for e in evs)
     b_ms = statistics.mean(e[1].elapsed_time(e[2]) for e in evs)
-    flops = 14.0 * B * H * T * T * D
+    # causal: the pairs above the diagonal do not exist, so half of the dense count is credited
+    flops = 14.0 * B * H * T * T * D * (0.5 if causal else 1.0)
     tot = f_ms + b_ms
-    # every bias element is read by the forward, the dQ and the dK/dV kernel, once per head it applies to
-    bias_gbs = None if bias is None else round(3.0 * B * H * T * T * bias.element_size() / tot / 1e6, 1)
-    cpu = cpu_extra(torch, "attention", B=B, T=T, H=H, D=D, dtype=dtype, bias=bias) if with_cpu else None
-    sdpa = torch_sdpa_case(torch, q, k, v, do, bias, flops) if with_cpu else None
+    cpu = cpu_extra(torch, "attention", B=B, T=T, H=H, D=D, dtype=dtype, bias=bias) if with_cpu and not causal else None
+    sdpa = torch_sdpa_case(torch, q, k, v, do, bias, flops) if with_cpu and not causal else None
     # roofline of the slower of the two calls (MFMA-bound; algorithmic FLOPs 4/14 forward, 10/14 backward)
     f_tf, b_tf = flops * 4 / 14 / f_ms / 1e9, flops * 10 / 14 / b_ms / 1e9
     slow_bwd = b_tf <= f_tf
@@ -387,7 +386,7 @@ def attention_case(torch, name, B, T, H, D, dtype, bias_kind, iters=20, with_cpu
             "frac": round((b_tf if slow_bwd else f_tf) / MFMA_PEAK_TFLOPS, 4),
             "avg_launch_ms": round(b_ms if slow_bwd else f_ms, 4),
             "duration_source": "HIP events around the call, mean of %d" % iters}
-    return {"workload": name, "roofline": roof, "cpu_baseline": cpu, "torch_sdpa": sdpa, "bias_read_gbs": bias_gbs, "fwd_ms": round(f_ms, 4), "bwd_ms": round(b_ms, 4),
+    return {"workload": name, "roofline": roof, "cpu_baseline": cpu, "torch_sdpa": sdpa, "bias_bytes": None if bias is None else bias.numel() * bias.element_size(), "fwd_ms": round(f_ms, 4), "bwd_ms": round(b_ms, 4),
             "tflops": round(flops / tot / 1e9, 2), "fwd_tflops": round(flops * 4 / 14 / f_ms / 1e9, 2),
             "bwd_tflops": round(flops * 10 / 14 / b_ms / 1e9, 2), "frac_mfma_peak": round(flops / tot / 1e9 / MFMA_PEAK_TFLOPS, 4)}
 
@@ -557,8 +556,13 @@ def extras(torch, only="", with_cpu=False):
         out.append(attention_case(torch, "attn_c5_zero: (2,4352,24,64) bf16 (B,1,T,T) bias of zeros", 2, 4352, 24, 64, bf, "zero_shared"))
     if only == "attn_c5_dense":
         out.append(attention_case(torch, "attn_c5_dense: (2,4352,24,64) bf16 (B,1,T,T) dense bias", 2, 4352, 24, 64, bf, "dense_shared"))
-    if only == "attn_c4_finite":
-        out.append(attention_case(torch, "attn_c4_finite: (2,2048,16,128) fp16 (B,H,T,T) finite bias", 2, 2048, 16, 128, torch.float16, "dense_full"))
+    # kernel quality at head dim 128 without the help of -inf blocks: a finite bias of config 4's shape, and a causal launch
+    if want("attn_c4_finite"):
+        out.append(attention_case(torch, "attn_c4_finite: (2,2048,16,128) fp16 (B,H,T,T) finite bias (no -inf blocks)", 2, 2048, 16, 128,
+                                  torch.float16, "dense_full"))
+    if want("attn_causal128"):
+        out.append(attention_case(torch, "attn_causal128: (2,8192,16,128) fp16 causal, no bias (FLOPs of the lower triangle)", 2, 8192, 16,
+                                  128, torch.float16, None, iters=10, causal=True))
     # buffer sets are sized so that their sum exceeds the 256 MB Infinity Cache
     if want("rms_c1"):
         out.append(rms_case(torch, "rms_c1: FusedRMSNorm (4,1024,1024) fp32 fwd+bwd", 4, [(1024, 1024)], torch.float32, 12, with_cpu=with_cpu))
@@ -618,20 +622,27 @@ def main():
                                "R=32, theta=10000, cutoff (2048,2048), P=2049",
                    "step": "rgd_ln_rope_qk_fwd + rgd_ln_rope_qk_bwd through the C ABI, 4 rotating buffer sets (1.07 GB)",
                    "algorithmic_bytes_per_step": step_bytes},
+        # achieved / frac: algorithmic bytes of a launch over the kernel's average duration in the committed rocprofv3
+        # kernel trace of this same command (reproducible: profiles/...), or over the live event figure when the summary is
+        # missing.  live_hip_events: the same launch timed in this run with an event before and after it; an event pair
+        # with nothing between costs `event_gap_ms`, and an interval holds between none and all of it, so the kernel's
+        # duration lies between the two figures given.
         "roofline": {"bound": "hbm", "kernel": "head_rows_kernel<bf16, LNROPE_BWD> (rgd_ln_rope_qk_bwd)",
-                     "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
-                     "algorithmic_bytes_per_launch": bwd_bytes, "avg_launch_ms": round(bwd_avg, 5),
-                     "duration_source": "HIP events recorded around every launch of the timed steps (a second pass over "
-                                        "the same steps), minus the event-to-event cost measured in that pass",
-                     "event_gap_ms_subtracted": round(event_gap, 5),
-                     # not measured by this run: the committed rocprofv3 summary of this same command
-                     "from_profile": {"file": PROFILE_SUMMARY, "measured_at": prof.get("measured_at"),
-                                      "traffic_bytes_per_launch": traffic, "rocprof_avg_launch_us": rocprof_us,
-                                      "frac_at_rocprof_duration": None if not rocprof_us else
-                                      round(bwd_bytes / rocprof_us / 1e3 / HBM_PEAK_GBS, 4)},
-                     "fwd_kernel": {"achieved": round(fwd_bytes / fwd_avg / 1e6, 1), "avg_launch_ms": round(fwd_avg, 5),
-                                    "frac": round(fwd_bytes / fwd_avg / 1e6 / HBM_PEAK_GBS, 4)}},
+                     "achieved": round(bwd_bytes / rocprof_us / 1e3 if rocprof_us else achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s",
+                     "frac": round((bwd_bytes / rocprof_us / 1e3 if rocprof_us else achieved) / HBM_PEAK_GBS, 4),
+                     "traffic": traffic, "algorithmic_bytes_per_launch": bwd_bytes,
+                     "avg_launch_ms": round(rocprof_us / 1e3 if rocprof_us else bwd_avg, 5),
+                     "duration_source": ("rocprofv3 --kernel-trace --stats of this command, " + PROFILE_SUMMARY +
+                                         " (measured at " + str(prof.get("measured_at")) + ")") if rocprof_us else
+                                        "HIP events of this run (no profile summary found)",
+                     "live_hip_events": {"interval_ms": round(bwd_avg + event_gap, 5), "event_gap_ms": round(event_gap, 5),
+                                         "frac_if_no_gap_inside": round(bwd_bytes / (bwd_avg + event_gap) / 1e6 / HBM_PEAK_GBS, 4),
+                                         "frac_if_whole_gap_inside": round(achieved / HBM_PEAK_GBS, 4),
+                                         "fwd_interval_ms": round(fwd_avg + event_gap, 5)},
+                     "fwd_kernel": {"rocprof_avg_launch_us": float(prof["rocprof_fwd_avg_launch_us"]) if "rocprof_fwd_avg_launch_us" in prof else None,
+                                    "frac": round(fwd_bytes / float(prof["rocprof_fwd_avg_launch_us"]) / 1e3 / HBM_PEAK_GBS, 4)
+                                    if "rocprof_fwd_avg_launch_us" in prof else None}},
         "timing": {"wall_ms_per_step": round(wall_ms, 5), "gpu_event_span_ms_per_step": round(gpu_ms, 5)},
     }
     if not args.skip_cpu:

@@ -285,7 +285,7 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
     // FAST (compile time): the tile is known to be full and on the 16-byte path.  The main loop runs on FAST steps
     // only; with the element-wise loader of ragged tiles in the same loop the compiler waits for every outstanding
     // load before a tile's first matrix instruction, and the prefetch hides nothing.
-    auto issue_loads = [&](int tile, auto FAST, auto SET) {
+    auto issue_loads = [&](int tile, auto FAST, auto SET) __attribute__((always_inline)) {
         u32x4(&kst)[LOADS] = kst_[PF2 ? decltype(SET)::value : 0];
         u32x4(&vst)[LOADS] = vst_[PF2 ? decltype(SET)::value : 0];
         const int key0 = tile * BN;
@@ -306,7 +306,7 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
             }
         }
     };
-    auto store_tiles = [&](int buf, auto SET) {
+    auto store_tiles = [&](int buf, auto SET) __attribute__((always_inline)) {
         u32x4(&kst)[LOADS] = kst_[PF2 ? decltype(SET)::value : 0];
         u32x4(&vst)[LOADS] = vst_[PF2 ? decltype(SET)::value : 0];
         if (padded) {
@@ -948,7 +948,7 @@ __global__ __launch_bounds__(BWD_THREADS, dkv_occupancy(DPAD, CLS ? BIAS_OFF : B
     bool row_st = false;                 // the row exists
     // FAST (compile time): all BQ query rows of the tile exist and the 16-byte path applies.  The main loop runs on
     // FAST steps only (see the dQ kernel).
-    auto issue_loads = [&](int tile, auto FAST) {
+    auto issue_loads = [&](int tile, auto FAST) __attribute__((always_inline)) {
         constexpr bool F = decltype(FAST)::value != 0;
         const int q0 = tile * BQ;
         const T* qt = qbase + (int64_t)q0 * p.q.sn;
@@ -978,7 +978,7 @@ __global__ __launch_bounds__(BWD_THREADS, dkv_occupancy(DPAD, CLS ? BIAS_OFF : B
             row_st = ok;
         }
     };
-    auto store_tiles = [&](int buf) {
+    auto store_tiles = [&](int buf) __attribute__((always_inline)) {
         T* qs = reinterpret_cast<T*>(smem_raw + buf * BUFB);
         T* ds = qs + TILE;
         float* st = reinterpret_cast<float*>(smem_raw + buf * BUFB + 2 * TILE * 2);
@@ -1008,7 +1008,7 @@ __global__ __launch_bounds__(BWD_THREADS, dkv_occupancy(DPAD, CLS ? BIAS_OFF : B
     const TB* bias_base = nullptr;  // bias of this batch and head (wavefront-uniform)
     uint32_t bias_lane_off = 0;     // this lane's key column, 16*g rows down
     BiasColumn<TB> bias_cur[NSUB], bias_nxt[NSUB];  // fetched one tile ahead of use
-    auto bias_load = [&](BiasColumn<TB> (&dst)[NSUB], int tile, auto FAST) {
+    auto bias_load = [&](BiasColumn<TB> (&dst)[NSUB], int tile, auto FAST) __attribute__((always_inline)) {
 #pragma unroll
         for (int u = 0; u < NSUB; ++u) {
             const int q0 = tile * BQ + u * 32;

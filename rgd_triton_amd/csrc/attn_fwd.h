@@ -185,15 +185,15 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
     constexpr bool REGULAR = ATTN_THREADS % CPR == 0;
     constexpr int ROWS_PER_PASS = ATTN_THREADS / CPR;
     const int ld_key0 = tid / CPR, ld_dc0 = tid % CPR;
-    auto chunk_key = [&](int i) { return REGULAR ? ld_key0 + i * ROWS_PER_PASS : (tid + i * ATTN_THREADS) / CPR; };
-    auto chunk_dc = [&](int i) { return REGULAR ? ld_dc0 : (tid + i * ATTN_THREADS) % CPR; };
+    auto chunk_key = [&](int i) __attribute__((always_inline)) { return REGULAR ? ld_key0 + i * ROWS_PER_PASS : (tid + i * ATTN_THREADS) / CPR; };
+    auto chunk_dc = [&](int i) __attribute__((always_inline)) { return REGULAR ? ld_dc0 : (tid + i * ATTN_THREADS) % CPR; };
     // element offsets of this thread's chunks inside a tile: one offset plus a uniform row step (REGULAR), or one
     // offset per chunk (head dim 96)
     // A head dim below the padded one (40, 80, 112, ...) leaves whole chunks past the end of a row: the fast
     // loader reads chunk 0 of the row in their place and store_tiles writes zeros.
     const bool padded = p.D != DPAD;
-    auto chunk_pad = [&](int i) { return chunk_dc(i) * 8 >= p.D; };  // recomputed where used: no register held
-    auto chunk_col = [&](int i) { return chunk_pad(i) ? 0 : chunk_dc(i) * 8; };
+    auto chunk_pad = [&](int i) __attribute__((always_inline)) { return chunk_dc(i) * 8 >= p.D; };  // recomputed where used: no register held
+    auto chunk_col = [&](int i) __attribute__((always_inline)) { return chunk_pad(i) ? 0 : chunk_dc(i) * 8; };
     const int koff0 = ld_key0 * (int)p.k.sn + chunk_col(0);
     const int voff0 = ld_key0 * (int)p.v.sn + chunk_col(0);
     int koff[REGULAR ? 1 : LOADS], voff[REGULAR ? 1 : LOADS];
@@ -213,7 +213,7 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
     // straight-line code.  The main loop below runs on FAST steps only: with the element-wise loader of ragged
     // tiles inside the same loop, the compiler has to wait for every outstanding load before a tile's first
     // matrix instruction (registers shared between the two loaders), and the prefetch hides nothing.
-    auto issue_loads = [&](int tile, auto FAST, auto SET) {
+    auto issue_loads = [&](int tile, auto FAST, auto SET) __attribute__((always_inline)) {
         u32x4(&kst)[LOADS] = kst_[PF2 ? decltype(SET)::value : 0];
         u32x4(&vst)[LOADS] = vst_[PF2 ? decltype(SET)::value : 0];
         const int key0 = tile * ATTN_BN;
@@ -240,7 +240,7 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
             }
         }
     };
-    auto store_tiles = [&](int buf, auto SET) {
+    auto store_tiles = [&](int buf, auto SET) __attribute__((always_inline)) {
         u32x4(&kst)[LOADS] = kst_[PF2 ? decltype(SET)::value : 0];
         u32x4(&vst)[LOADS] = vst_[PF2 ? decltype(SET)::value : 0];
         if (padded) {
