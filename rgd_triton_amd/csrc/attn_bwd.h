@@ -260,11 +260,18 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
         }
     }
 
+    // scalars the loop works with: copies of their own (see own_scalar)
+    struct {
+        int64_t ksn, vsn;
+        int Tk, Tq, D, causal;
+        float scale_log2;
+    } L = {own_scalar(p.k.sn), own_scalar(p.v.sn), own_scalar(p.Tk), own_scalar(p.Tq), own_scalar(p.D), own_scalar(p.causal),
+           own_scalar(p.scale_log2)};
     const T* kbase = static_cast<const T*>(p.k.ptr) + b * p.k.sb + h * p.k.sh;
     const T* vbase = static_cast<const T*>(p.v.ptr) + b * p.v.sb + h * p.v.sh;
     // A head dim below the padded one (40, 80, 112, ...) leaves whole chunks past the end of a row: the fast loader
     // reads chunk 0 of the row in their place and store_tiles writes zeros (pad_mask bit i = chunk i).
-    const bool padded = p.D != DPAD;
+    const bool padded = L.D != DPAD;
     uint32_t pad_mask = 0;
     int ld_key[LOADS], ld_dc[LOADS], koff[LOADS], voff[LOADS], soff[LOADS];
 #pragma unroll
@@ -272,10 +279,10 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
         const int id = tid + i * BWD_THREADS;
         ld_key[i] = id / CPR;
         ld_dc[i] = id % CPR;
-        const bool pad = ld_dc[i] * 8 >= p.D;
+        const bool pad = ld_dc[i] * 8 >= L.D;
         pad_mask |= (pad ? 1u : 0u) << i;
-        koff[i] = ld_key[i] * (int)p.k.sn + (pad ? 0 : ld_dc[i] * 8);
-        voff[i] = ld_key[i] * (int)p.v.sn + (pad ? 0 : ld_dc[i] * 8);
+        koff[i] = ld_key[i] * (int)L.ksn + (pad ? 0 : ld_dc[i] * 8);
+        voff[i] = ld_key[i] * (int)L.vsn + (pad ? 0 : ld_dc[i] * 8);
         soff[i] = ld_key[i] * ST + ld_dc[i] * 8;
     }
     const bool fast_tiles = vec;  // rows made of whole 16-byte chunks
@@ -289,9 +296,9 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
         u32x4(&kst)[LOADS] = kst_[PF2 ? decltype(SET)::value : 0];
         u32x4(&vst)[LOADS] = vst_[PF2 ? decltype(SET)::value : 0];
         const int key0 = tile * BN;
-        const T* kt = kbase + (int64_t)key0 * p.k.sn;
-        const T* vt = vbase + (int64_t)key0 * p.v.sn;
-        if (decltype(FAST)::value || (fast_tiles && key0 + BN <= p.Tk)) {
+        const T* kt = kbase + (int64_t)key0 * L.ksn;
+        const T* vt = vbase + (int64_t)key0 * L.vsn;
+        if (decltype(FAST)::value || (fast_tiles && key0 + BN <= L.Tk)) {
 #pragma unroll
             for (int i = 0; i < LOADS; ++i) {
                 kst[i] = *reinterpret_cast<const u32x4*>(kt + koff[i]);
@@ -300,9 +307,9 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
         } else {
 #pragma unroll
             for (int i = 0; i < LOADS; ++i) {
-                const bool ok = key0 + ld_key[i] < p.Tk;
-                kst[i] = load8<T>(kt + (int64_t)ld_key[i] * p.k.sn, ld_dc[i] * 8, p.D, ok, vec);
-                vst[i] = load8<T>(vt + (int64_t)ld_key[i] * p.v.sn, ld_dc[i] * 8, p.D, ok, vec);
+                const bool ok = key0 + ld_key[i] < L.Tk;
+                kst[i] = load8<T>(kt + (int64_t)ld_key[i] * L.ksn, ld_dc[i] * 8, L.D, ok, vec);
+                vst[i] = load8<T>(vt + (int64_t)ld_key[i] * L.vsn, ld_dc[i] * 8, L.D, ok, vec);
             }
         }
     };
@@ -332,7 +339,7 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
     }
     const uint8_t* const cls_lds = smem_raw + DqSmem<DPAD>::BYTES;  // CLS: class of every key tile for the workgroup's 128 rows
     if constexpr (CLS)
-        cls_tiles_to_lds(p.cls, b, qb * (BWD_BM / CLS_ROWS), BWD_BM / CLS_ROWS, (p.Tk + BN - 1) / BN, smem_raw + DqSmem<DPAD>::BYTES, tid);
+        cls_tiles_to_lds(p.cls, b, qb * (BWD_BM / CLS_ROWS), BWD_BM / CLS_ROWS, (L.Tk + BN - 1) / BN, smem_raw + DqSmem<DPAD>::BYTES, tid);
     int run_end = t_end;  // end of the run of tiles that is being worked on (all of them unless CLS)
     // CLS: class of the tile of the next step, read from the table in LDS a step ahead (in a register of every lane; the
     // step makes a scalar of it)
@@ -350,12 +357,12 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
         constexpr int AH = decltype(AHEAD)::value;
         const int buf = j & 1;
         const int key0 = j * BN;
-        const bool tail = !F && key0 + BN > p.Tk;
+        const bool tail = !F && key0 + BN > L.Tk;
         if (F || j + 1 < run_end) {
             if constexpr (AH == 0) issue_loads(j + 1, FAST, IntC<0>{});
             else issue_loads(j + 2, FAST, IntC<AH - 1>{});
             if constexpr (BIAS_AHEAD)
-                bias_nxt.load(bias_row, key0 + BN, g, p.Tk, F || (p.bias_vec && key0 + 2 * BN <= p.Tk));
+                bias_nxt.load(bias_row, key0 + BN, g, L.Tk, F || (p.bias_vec && key0 + 2 * BN <= L.Tk));
         }
         // WB: the tile has a bias: the registers fetched a step ago, or (CLS: a run of MIXED tiles, which are few) read
         // here, at the start of the tile's own step
@@ -389,41 +396,55 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
                 for (int v = 0; v < 16; ++v) dp[kb][v] = 0.f;
             }
         }
+        auto products = [&]() __attribute__((always_inline)) {
 #pragma unroll
-        for (int kb = 0; kb < NKB; ++kb)
+            for (int kb = 0; kb < NKB; ++kb) {
 #pragma unroll
-            for (int v = 0; v < 16; ++v) s[kb][v] = 0.f;
+                for (int c = 0; c < NC; ++c) {
+                    const u32x4 ka = *reinterpret_cast<const u32x4*>(ks + kb * 32 * ST + c * 16);
+                    s[kb] = MM::run(as_v8<T>(ka), qreg[c], s[kb]);
+                    const u32x4 va = *reinterpret_cast<const u32x4*>(vs + kb * 32 * ST + c * 16);
+                    dp[kb] = MM::run(as_v8<T>(va), doreg[c], dp[kb]);
+                }
+            }
+        };
+        auto from_zero = [&]() __attribute__((always_inline)) {
+#pragma unroll
+            for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) s[kb][v] = 0.f;
+            products();
+        };
         if constexpr (CLS) {
             // A MIXED or COLUMN tile (few; tc is its class): the first product starts from the bias, in units of the raw
             // scores, instead of from zero, and the tile goes on like every other tile.  The bias is read here, straight
             // into the accumulators: no register is held for it while other tiles run, and the row address is formed here
             // for the same reason.  COLUMN: every row of the tile is the first row of this wavefront's 32, which all its
-            // lanes read.
+            // lanes read.  The products are written out twice, so that the one that starts from zero keeps its zero inside
+            // its first matrix instructions instead of in 32 registers that something has to clear.
             if (__builtin_expect(tc != CLS_ZERO, 0)) {
-            int row = tc == CLS_COLUMN ? min(qb * BWD_BM + wave * 32, p.Tq - 1) : q_ld;
-            asm volatile("" : "+v"(row));
-            const TB* here = static_cast<const TB*>(p.bias.ptr) + b * p.bias.sb + h * p.bias.sh + (int64_t)row * p.bias.sn;
-            const float per_score = kLog2e / p.scale_log2;
+                int row = tc == CLS_COLUMN ? min(qb * BWD_BM + wave * 32, L.Tq - 1) : q_ld;
+                asm volatile("" : "+v"(row));
+                // the bias tensor is read from the kernel's argument memory here, not kept in scalar registers through the loop
+                const AttnTensor& bt = cold_params<AttnBwdParams>().bias;
+                const TB* here = static_cast<const TB*>(bt.ptr) + b * bt.sb + h * bt.sh + (int64_t)row * bt.sn;
+                const float per_score = kLog2e / L.scale_log2;
 #pragma unroll
-            for (int kb = 0; kb < NKB; ++kb) {
-                BiasRuns<TB, 1> half;
-                half.load(here, key0 + kb * 32, g, p.Tk, key0 + BN <= p.Tk);
-                float bias_h[16];
-                half.decode_run(0, bias_h);
+                for (int kb = 0; kb < NKB; ++kb) {
+                    BiasRuns<TB, 1> half;
+                    half.load(here, key0 + kb * 32, g, L.Tk, key0 + BN <= L.Tk);
+                    float bias_h[16];
+                    half.decode_run(0, bias_h);
 #pragma unroll
-                for (int v = 0; v < 16; ++v) s[kb][v] = bias_h[v] * per_score;
+                    for (int v = 0; v < 16; ++v) s[kb][v] = bias_h[v] * per_score;
+                }
+                products();
+                asm volatile("" ::: "memory");  // (keeps the two copies apart)
+            } else {
+                from_zero();
             }
-            }
-        }
-#pragma unroll
-        for (int kb = 0; kb < NKB; ++kb) {
-#pragma unroll
-            for (int c = 0; c < NC; ++c) {
-                const u32x4 ka = *reinterpret_cast<const u32x4*>(ks + kb * 32 * ST + c * 16);
-                s[kb] = MM::run(as_v8<T>(ka), qreg[c], s[kb]);
-                const u32x4 va = *reinterpret_cast<const u32x4*>(vs + kb * 32 * ST + c * 16);
-                dp[kb] = MM::run(as_v8<T>(va), doreg[c], dp[kb]);
-            }
+        } else {
+            from_zero();
         }
         }
 #if !RGD_DQ_SKIP_EARLY
@@ -445,19 +466,19 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     if constexpr (WITH_BIAS && !CLS)
-                        s[kb][v] = fmaf(s[kb][v], p.scale_log2, fmaf(bias_v[kb][v], kLog2e, neg_lse_l2));
+                        s[kb][v] = fmaf(s[kb][v], L.scale_log2, fmaf(bias_v[kb][v], kLog2e, neg_lse_l2));
                     else
-                        s[kb][v] = fmaf(s[kb][v], p.scale_log2, neg_lse_l2);
+                        s[kb][v] = fmaf(s[kb][v], L.scale_log2, neg_lse_l2);
                 }
         }
-        const bool diag = p.causal && (key0 + BN - 1 > qb * BWD_BM + wave * 32);
+        const bool diag = L.causal && (key0 + BN - 1 > qb * BWD_BM + wave * 32);
         if (tail || diag) {
 #pragma unroll
             for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     const int key = key0 + kb * 32 + g * 16 + v;
-                    if (key >= p.Tk || (p.causal && key > q_row)) s[kb][v] = -INFINITY;
+                    if (key >= L.Tk || (L.causal && key > q_row)) s[kb][v] = -INFINITY;
                 }
         }
         uint32_t dsk[NKB][8];
@@ -545,12 +566,12 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
         if (rb < re) {
             issue_loads(rb, IntC<0>{}, IntC<0>{});
             store_tiles(rb & 1, IntC<0>{});
-            if constexpr (BIAS_AHEAD) bias_cur.load(bias_row, rb * BN, g, p.Tk, p.bias_vec && (rb + 1) * BN <= p.Tk);
+            if constexpr (BIAS_AHEAD) bias_cur.load(bias_row, rb * BN, g, L.Tk, p.bias_vec && (rb + 1) * BN <= L.Tk);
         }
         __syncthreads();
         // tiles below n_fast are full and take the 16-byte path; a FAST step also prefetches tile j+1
         const bool fast_ok = fast_tiles && (!HAS_BIAS || p.bias_vec);
-        const int n_fast = fast_ok ? min(re, p.Tk / BN) : rb;
+        const int n_fast = fast_ok ? min(re, L.Tk / BN) : rb;
         int j = rb;
         if constexpr (PF2) {
             if (n_fast - j >= 4) {
@@ -590,6 +611,9 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
         run_tiles(t_begin, t_end, IntC<(HAS_BIAS ? 1 : 0)>{});
     }
 
+    // CLS: what only the epilogue needs is read from the kernel's argument memory here instead of sitting in scalar
+    // registers through the loop, which has none to spare
+    const AttnBwdParams& pe = CLS ? cold_params<AttnBwdParams>() : p;
     if constexpr (RECORD) {
         if (p.ranges != nullptr && lane == 0 && item.part == 0) {
             // a part of a split item has seen a part of the keys: its rows are noted as having all of them
@@ -600,15 +624,15 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
         }
     }
     if (item.nparts > 1) {  // part of a split item: leave the unscaled fp32 sums
-        float* row = p.part + ((int64_t)item.part_id * BWD_BM + wave * 32 + li) * DPAD;
+        float* row = pe.part + ((int64_t)item.part_id * BWD_BM + wave * 32 + li) * DPAD;
 #pragma unroll
         for (int d = 0; d < NDB; ++d) store_part16(row, d * 32 + g * 16, acc[d]);
         return;
     }
     if (q_valid) {
-        T* dqp = static_cast<T*>(const_cast<void*>(p.dq.ptr)) + b * p.dq.sb + h * p.dq.sh + (int64_t)q_row * p.dq.sn;
+        T* dqp = static_cast<T*>(const_cast<void*>(pe.dq.ptr)) + b * pe.dq.sb + h * pe.dq.sh + (int64_t)q_row * pe.dq.sn;
 #pragma unroll
-        for (int d = 0; d < NDB; ++d) store_row16<T>(dqp, d * 32 + g * 16, p.D, vec, acc[d], p.scale);
+        for (int d = 0; d < NDB; ++d) store_row16<T>(dqp, d * 32 + g * 16, pe.D, vec, acc[d], pe.scale);
     }
 }
 

@@ -149,7 +149,6 @@ __global__ __launch_bounds__(256) void attn_bias_classify_kernel(const TB* __res
     constexpr int EPC = 16 / (int)sizeof(TB);      // elements per 16-byte chunk
     constexpr int NLD = 512 / (64 * EPC);          // load instructions per row of the strip (1 or 2)
     constexpr int LPT = CLS_KEYS / EPC;            // lanes per tile (8 or 16)
-    constexpr int ROWS = 16 / NLD;                 // rows in flight
     constexpr uint32_t PAT = NegInfBits<TB>::value;
     const int lane = threadIdx.x & 63;
     const int w = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -178,22 +177,25 @@ __global__ __launch_bounds__(256) void attn_bias_classify_kernel(const TB* __res
         return m & (LPT == 16 ? 0x0001000100010001ull : 0x0101010101010101ull);
     };
     uint64_t zero_t[NLD], neg_t[NLD], col_t[NLD];
-    for (int r0 = 0; r0 < CLS_ROWS; r0 += ROWS) {
-        u32x4 v[ROWS][NLD];
+    // rows [r0, r0 + N) of the strip, all their loads in flight at once; returns whether any tile may still be something
+    // other than MIXED
+    auto rows = [&](auto R0, auto N) __attribute__((always_inline)) {
+        constexpr int r0 = decltype(R0)::value, n = decltype(N)::value;
+        u32x4 v[n][NLD];
 #pragma unroll
-        for (int r = 0; r < ROWS; ++r) {
+        for (int r = 0; r < n; ++r) {
             const int row = min(row32 * CLS_ROWS + r0 + r, Tq - 1);
 #pragma unroll
             for (int i = 0; i < NLD; ++i) v[r][i] = *reinterpret_cast<const u32x4*>(base + (int64_t)row * sn + key[i]);
         }
 #pragma unroll
-        for (int r = 0; r < ROWS; ++r)
+        for (int r = 0; r < n; ++r)
 #pragma unroll
             for (int i = 0; i < NLD; ++i) {
                 all_and[i] &= v[r][i];
                 all_or[i] |= v[r][i];
             }
-        uint64_t open = 0;  // tiles that may still be something other than MIXED
+        uint64_t open = 0;
 #pragma unroll
         for (int i = 0; i < NLD; ++i) {
             const uint32_t a = all_and[i][0] & all_and[i][1] & all_and[i][2] & all_and[i][3];
@@ -205,7 +207,16 @@ __global__ __launch_bounds__(256) void attn_bias_classify_kernel(const TB* __res
             col_t[i] = fold(__builtin_amdgcn_ballot_w64(ok[i] && same));
             open |= col_t[i];  // a ZERO or NEG tile is a COLUMN tile too
         }
-        if (open == 0) break;
+        return open != 0;
+    };
+    // two rows tell a dense bias from a mask (two rows of a dense bias differ in every tile): the strip is left after
+    // them; otherwise the other thirty rows follow, all their loads in flight at once
+    if (rows(IntC<0>{}, IntC<2>{})) {
+        if constexpr (NLD == 1) {
+            rows(IntC<2>{}, IntC<CLS_ROWS - 2>{});
+        } else {
+            if (rows(IntC<2>{}, IntC<14>{})) rows(IntC<16>{}, IntC<16>{});
+        }
     }
     if (lane == 0) {
         uint32_t code = 0;

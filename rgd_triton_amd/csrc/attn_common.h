@@ -331,5 +331,30 @@ inline AttnSplit attn_split_plan(int64_t items, int cus, int per_cu, int inner_t
     return plan;
 }
 
+// A copy of a scalar (wavefront-uniform) value that the compiler treats as a value of its own.  The kernels receive their
+// parameters as one struct, which arrives in groups of 8 or 16 scalar registers; a field that a loop uses keeps its whole
+// group alive, and when scalar registers run short the compiler parks and fetches whole groups (16 lane reads per step
+// for one stride).  Loop code therefore works on copies made with this function before the loop.
+template <typename X> __device__ __forceinline__ X own_scalar(X v) {
+    // a real move into a new register: an empty statement with a tied operand would be folded back into the group
+    static_assert(sizeof(X) == 4 || sizeof(X) == 8, "own_scalar: 32- or 64-bit values");
+    X r;
+    if constexpr (sizeof(X) == 4)
+        asm volatile("s_mov_b32 %0, %1" : "=s"(r) : "s"(v));
+    else
+        asm volatile("s_mov_b64 %0, %1" : "=s"(r) : "s"(v));
+    return r;
+}
+
+// The kernel's parameter struct as it lies in argument memory (the kernels take one struct, by value, as their first
+// argument), for code that runs rarely: a field read through this reference is loaded where it is used, instead of
+// sitting in a scalar register through every loop of the kernel.  (The empty asm keeps the compiler from moving the
+// loads out of the rarely executed block they are written in.)
+template <typename P> __device__ __forceinline__ const P& cold_params() {
+    auto ka = __builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(ka));
+    return *(const P*)ka;
+}
+
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;

@@ -178,6 +178,13 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
     constexpr int TASKS = ATTN_BN * CPR;
     static_assert(TASKS % ATTN_THREADS == 0, "tile chunks must divide evenly over the workgroup");
     constexpr int LOADS = TASKS / ATTN_THREADS;
+    // scalars the loop works with: copies of their own (see own_scalar)
+    struct {
+        int64_t ksn, vsn;
+        int Tk, Tq, D, causal;
+        float scale_log2;
+    } L = {own_scalar(p.k.sn), own_scalar(p.v.sn), own_scalar(p.Tk), own_scalar(p.Tq), own_scalar(p.D), own_scalar(p.causal),
+           own_scalar(p.scale_log2)};
     const T* kbase = static_cast<const T*>(p.k.ptr) + b * p.k.sb + h * p.k.sh;
     const T* vbase = static_cast<const T*>(p.v.ptr) + b * p.v.sb + h * p.v.sh;
     // chunk i of this thread is row (ld_key0 + i*ROWS_PER_PASS) when the row length divides the
@@ -191,21 +198,21 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
     // offset per chunk (head dim 96)
     // A head dim below the padded one (40, 80, 112, ...) leaves whole chunks past the end of a row: the fast
     // loader reads chunk 0 of the row in their place and store_tiles writes zeros.
-    const bool padded = p.D != DPAD;
-    auto chunk_pad = [&](int i) __attribute__((always_inline)) { return chunk_dc(i) * 8 >= p.D; };  // recomputed where used: no register held
+    const bool padded = L.D != DPAD;
+    auto chunk_pad = [&](int i) __attribute__((always_inline)) { return chunk_dc(i) * 8 >= L.D; };  // recomputed where used: no register held
     auto chunk_col = [&](int i) __attribute__((always_inline)) { return chunk_pad(i) ? 0 : chunk_dc(i) * 8; };
-    const int koff0 = ld_key0 * (int)p.k.sn + chunk_col(0);
-    const int voff0 = ld_key0 * (int)p.v.sn + chunk_col(0);
+    const int koff0 = ld_key0 * (int)L.ksn + chunk_col(0);
+    const int voff0 = ld_key0 * (int)L.vsn + chunk_col(0);
     int koff[REGULAR ? 1 : LOADS], voff[REGULAR ? 1 : LOADS];
     if constexpr (!REGULAR) {
 #pragma unroll
         for (int i = 0; i < LOADS; ++i) {
-            koff[i] = chunk_key(i) * (int)p.k.sn + chunk_col(i);
-            voff[i] = chunk_key(i) * (int)p.v.sn + chunk_col(i);
+            koff[i] = chunk_key(i) * (int)L.ksn + chunk_col(i);
+            voff[i] = chunk_key(i) * (int)L.vsn + chunk_col(i);
         }
     }
     // rows made of whole 16-byte chunks: straight-line loads, no masking except in the last tile
-    const bool fast_tiles = vec && p.D % 8 == 0;
+    const bool fast_tiles = vec && L.D % 8 == 0;
     // two staging register sets when the main loop fetches two tiles ahead (PF2), else one
     constexpr bool PF2 = RGD_FWD_PREFETCH2 && DPAD <= 64 && (!HAS_BIAS || RGD_FWD_PREFETCH2_BIAS) && (!CLS || RGD_CLS_FWD_PF2);
     u32x4 kst_[PF2 ? 2 : 1][LOADS], vst_[PF2 ? 2 : 1][LOADS];
@@ -217,14 +224,14 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
         u32x4(&kst)[LOADS] = kst_[PF2 ? decltype(SET)::value : 0];
         u32x4(&vst)[LOADS] = vst_[PF2 ? decltype(SET)::value : 0];
         const int key0 = tile * ATTN_BN;
-        const T* kt = kbase + (int64_t)key0 * p.k.sn;
-        const T* vt = vbase + (int64_t)key0 * p.v.sn;
-        if (decltype(FAST)::value || (fast_tiles && key0 + ATTN_BN <= p.Tk)) {
+        const T* kt = kbase + (int64_t)key0 * L.ksn;
+        const T* vt = vbase + (int64_t)key0 * L.vsn;
+        if (decltype(FAST)::value || (fast_tiles && key0 + ATTN_BN <= L.Tk)) {
 #pragma unroll
             for (int i = 0; i < LOADS; ++i) {  // wavefront-uniform tile base + fixed per-thread offset
                 if constexpr (REGULAR) {
-                    kst[i] = *reinterpret_cast<const u32x4*>(kt + (int64_t)(i * ROWS_PER_PASS) * p.k.sn + koff0);
-                    vst[i] = *reinterpret_cast<const u32x4*>(vt + (int64_t)(i * ROWS_PER_PASS) * p.v.sn + voff0);
+                    kst[i] = *reinterpret_cast<const u32x4*>(kt + (int64_t)(i * ROWS_PER_PASS) * L.ksn + koff0);
+                    vst[i] = *reinterpret_cast<const u32x4*>(vt + (int64_t)(i * ROWS_PER_PASS) * L.vsn + voff0);
                 } else {
                     kst[i] = *reinterpret_cast<const u32x4*>(kt + koff[i]);
                     vst[i] = *reinterpret_cast<const u32x4*>(vt + voff[i]);
@@ -234,9 +241,9 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
 #pragma unroll
             for (int i = 0; i < LOADS; ++i) {
                 const int key = chunk_key(i), dc = chunk_dc(i);
-                const bool ok = key0 + key < p.Tk;
-                kst[i] = load8<T>(kt + (int64_t)key * p.k.sn, dc * 8, p.D, ok, vec);
-                vst[i] = load8<T>(vt + (int64_t)key * p.v.sn, dc * 8, p.D, ok, vec);
+                const bool ok = key0 + key < L.Tk;
+                kst[i] = load8<T>(kt + (int64_t)key * L.ksn, dc * 8, L.D, ok, vec);
+                vst[i] = load8<T>(vt + (int64_t)key * L.vsn, dc * 8, L.D, ok, vec);
             }
         }
     };
@@ -268,7 +275,7 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
     if constexpr (HAS_BIAS && !CLS)
         bias_row = static_cast<const TB*>(p.bias.ptr) + b * p.bias.sb + h * p.bias.sh + (int64_t)q_ld * p.bias.sn;
     if constexpr (CLS)
-        cls_tiles_to_lds(p.cls, b, qb * (ATTN_BM / CLS_ROWS), ATTN_BM / CLS_ROWS, (p.Tk + ATTN_BN - 1) / ATTN_BN, smem_raw + SM::BYTES, tid);
+        cls_tiles_to_lds(p.cls, b, qb * (ATTN_BM / CLS_ROWS), ATTN_BM / CLS_ROWS, (L.Tk + ATTN_BN - 1) / ATTN_BN, smem_raw + SM::BYTES, tid);
     int run_end = t_end;  // end of the run of tiles that is being worked on (all of them unless CLS)
     // CLS: class of the tile of the next step, read from the table in LDS a step ahead (in a register of every lane; the
     // step makes a scalar of it)
@@ -284,12 +291,12 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
         constexpr int AH = decltype(AHEAD)::value;
         const int buf = j & 1;
         const int key0 = j * ATTN_BN;
-        const bool tail = !F && key0 + ATTN_BN > p.Tk;
+        const bool tail = !F && key0 + ATTN_BN > L.Tk;
         if (F || j + 1 < run_end) {
             if constexpr (AH == 0) issue_loads(j + 1, FAST, IntC<0>{});
             else issue_loads(j + 2, FAST, IntC<AH - 1>{});
             if constexpr (BIAS_AHEAD)
-                bias_nxt.load(bias_row, key0 + ATTN_BN, g, p.Tk, F || (p.bias_vec && key0 + 2 * ATTN_BN <= p.Tk));
+                bias_nxt.load(bias_row, key0 + ATTN_BN, g, L.Tk, F || (p.bias_vec && key0 + 2 * ATTN_BN <= L.Tk));
         }
         if constexpr (!SPLIT_HALVES) {
             // d <= 64: both 32-key halves of the tile go through the softmax together.
@@ -301,41 +308,56 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
             // ---- S^T = K . Q^T ----
             const T* ks = ks_base + buf * TILE + a_off;
             f32x16 s[2];
+            // the two halves alternate, so consecutive matrix instructions never wait for each other's result
+            auto products = [&]() __attribute__((always_inline)) {
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+                for (int c = 0; c < NC; ++c)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) s[kb][v] = 0.f;
+                    for (int kb = 0; kb < 2; ++kb) {
+                        const u32x4 a = *reinterpret_cast<const u32x4*>(ks + kb * 32 * ST + c * 16);
+                        s[kb] = MM::run(as_v8<T>(a), qreg[c], s[kb]);
+                    }
+            };
+            auto from_zero = [&]() __attribute__((always_inline)) {
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) s[kb][v] = 0.f;
+                products();
+            };
             if constexpr (CLS) {
                 // A MIXED or COLUMN tile (few; tc is its class): the product starts from the bias, in units of the raw
                 // scores, instead of from zero, and the tile goes on like every other tile.  The bias is read here, straight
                 // into the accumulators: no register is held for it while other tiles run, and the row address is formed
                 // here for the same reason.  COLUMN: every row of the tile is the first row of this wavefront's 32, which
-                // all its lanes read.  (A copy of the whole step for these tiles, which would leave the step of the other
-                // tiles exactly that of the kernel without bias, costs that step registers it does not have: spills.)
+                // all its lanes read.  The product is written out twice, so that the one that starts from zero keeps its
+                // zero inside its first matrix instructions instead of in 32 registers that something has to clear.
+                // (A copy of the whole step for these tiles, which would leave the step of the other tiles exactly that of
+                // the kernel without bias, costs that step registers it does not have: spills.)
                 if (__builtin_expect(tc != CLS_ZERO, 0)) {
-                int row = tc == CLS_COLUMN ? min(qb * ATTN_BM + wave * 32, p.Tq - 1) : q_ld;
-                asm volatile("" : "+v"(row));
-                const TB* here = static_cast<const TB*>(p.bias.ptr) + b * p.bias.sb + h * p.bias.sh + (int64_t)row * p.bias.sn;
-                const float per_score = kLog2e / p.scale_log2;
+                    int row = tc == CLS_COLUMN ? min(qb * ATTN_BM + wave * 32, L.Tq - 1) : q_ld;
+                    asm volatile("" : "+v"(row));
+                    // the bias tensor is read from the kernel's argument memory here, not kept in scalar registers through the loop
+                    const AttnTensor& bt = cold_params<AttnFwdParams>().bias;
+                    const TB* here = static_cast<const TB*>(bt.ptr) + b * bt.sb + h * bt.sh + (int64_t)row * bt.sn;
+                    const float per_score = kLog2e / L.scale_log2;
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb) {
-                    BiasRuns<TB, 1> half;
-                    half.load(here, key0 + kb * 32, g, p.Tk, key0 + ATTN_BN <= p.Tk);
-                    float bias_v[16];
-                    half.decode_run(0, bias_v);
+                    for (int kb = 0; kb < 2; ++kb) {
+                        BiasRuns<TB, 1> half;
+                        half.load(here, key0 + kb * 32, g, L.Tk, key0 + ATTN_BN <= L.Tk);
+                        float bias_v[16];
+                        half.decode_run(0, bias_v);
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) s[kb][v] = bias_v[v] * per_score;
+                        for (int v = 0; v < 16; ++v) s[kb][v] = bias_v[v] * per_score;
+                    }
+                    products();
+                    asm volatile("" ::: "memory");  // (keeps the two copies apart)
+                } else {
+                    from_zero();
                 }
-                }
+            } else {
+                from_zero();
             }
-            // the two halves alternate, so consecutive matrix instructions never wait for each other's result
-#pragma unroll
-            for (int c = 0; c < NC; ++c)
-#pragma unroll
-                for (int kb = 0; kb < 2; ++kb) {
-                    const u32x4 a = *reinterpret_cast<const u32x4*>(ks + kb * 32 * ST + c * 16);
-                    s[kb] = MM::run(as_v8<T>(a), qreg[c], s[kb]);
-                }
 
             // ---- t = logit - m_ref (log2 domain) ----
             const float m_off = m_ref == -INFINITY ? 0.f : m_ref;
@@ -345,13 +367,13 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
                     float bias_v[16];
                     bias_use.decode_run(kb, bias_v);
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) s[kb][v] = fmaf(s[kb][v], p.scale_log2, fmaf(bias_v[v], kLog2e, -m_off));
+                    for (int v = 0; v < 16; ++v) s[kb][v] = fmaf(s[kb][v], L.scale_log2, fmaf(bias_v[v], kLog2e, -m_off));
                 } else {
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) s[kb][v] = fmaf(s[kb][v], p.scale_log2, -m_off);
+                    for (int v = 0; v < 16; ++v) s[kb][v] = fmaf(s[kb][v], L.scale_log2, -m_off);
                 }
             }
-            const bool diag = p.causal && (key0 + ATTN_BN - 1 > qb * ATTN_BM + wave * 32);
+            const bool diag = L.causal && (key0 + ATTN_BN - 1 > qb * ATTN_BM + wave * 32);
             // running maximum of the tile and, if needed, a move of the reference exponent (first finite logit of
             // the row, or growth > 2^8): rescales the accumulators and shifts the logits
             auto max_and_move = [&]() __attribute__((always_inline)) {
@@ -420,7 +442,7 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
 #pragma unroll
                         for (int v = 0; v < 16; ++v) {
                             const int key = key0 + kb * 32 + g * 16 + v;
-                            if (key >= p.Tk || (p.causal && key > q_row)) s[kb][v] = -INFINITY;
+                            if (key >= L.Tk || (L.causal && key > q_row)) s[kb][v] = -INFINITY;
                         }
                 }
                 max_and_move();
@@ -450,7 +472,7 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
             // Each 32-key half of the tile is a complete softmax step of its own (S -> p -> PV), so only 16
             // logits are live at a time; the register budget buys wavefronts per SIMD, and those hide the
             // LDS and matrix-pipe latencies of one another.
-            const bool diag = p.causal && (key0 + ATTN_BN - 1 > qb * ATTN_BM + wave * 32);
+            const bool diag = L.causal && (key0 + ATTN_BN - 1 > qb * ATTN_BM + wave * 32);
             const T* ks = ks_base + buf * TILE + a_off;
             const T* vs = vs_base + buf * TILE + tr_off;
 #pragma unroll
@@ -482,16 +504,16 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
                     float bias_v[16];
                     bias_cur.decode_run(kb, bias_v);
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) s[v] = fmaf(s[v], p.scale_log2, fmaf(bias_v[v], kLog2e, -m_off));
+                    for (int v = 0; v < 16; ++v) s[v] = fmaf(s[v], L.scale_log2, fmaf(bias_v[v], kLog2e, -m_off));
                 } else {
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) s[v] = fmaf(s[v], p.scale_log2, -m_off);
+                    for (int v = 0; v < 16; ++v) s[v] = fmaf(s[v], L.scale_log2, -m_off);
                 }
                 if (tail || diag) {
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
                         const int key = key0 + kb * 32 + g * 16 + v;
-                        if (key >= p.Tk || (p.causal && key > q_row)) s[v] = -INFINITY;
+                        if (key >= L.Tk || (L.causal && key > q_row)) s[v] = -INFINITY;
                     }
                 }
                 float tmax = -INFINITY;
@@ -553,9 +575,13 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
     // CLS: the class of the tile goes into the step as a scalar (read from LDS a step ahead)
     auto step = [&](const int j, auto FAST, auto AHEAD, auto WBIAS) __attribute__((always_inline)) {
         if constexpr (CLS) {
+#ifdef RGD_CLS_DEBUG_NOCHECK
+            tile_step(j, FAST, AHEAD, IntC<0>{}, CLS_ZERO);
+#else
             const int tc = __builtin_amdgcn_readfirstlane(cls_ahead);
             cls_ahead = cls_lds[min(j + 1, CLS_LDS_BYTES - 1)];
             tile_step(j, FAST, AHEAD, IntC<0>{}, tc);
+#endif
         } else {
             tile_step(j, FAST, AHEAD, WBIAS, 0);
         }
@@ -568,12 +594,12 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
         if (rb < re) {
             issue_loads(rb, IntC<0>{}, IntC<0>{});
             store_tiles(rb & 1, IntC<0>{});
-            if constexpr (BIAS_AHEAD) bias_cur.load(bias_row, rb * ATTN_BN, g, p.Tk, p.bias_vec && (rb + 1) * ATTN_BN <= p.Tk);
+            if constexpr (BIAS_AHEAD) bias_cur.load(bias_row, rb * ATTN_BN, g, L.Tk, p.bias_vec && (rb + 1) * ATTN_BN <= L.Tk);
         }
         __syncthreads();
         // tiles below n_fast are full and take the 16-byte path; a FAST step also prefetches tile j+1
         const bool fast_ok = fast_tiles && (!HAS_BIAS || p.bias_vec);
-        const int n_fast = fast_ok ? min(re, p.Tk / ATTN_BN) : rb;
+        const int n_fast = fast_ok ? min(re, L.Tk / ATTN_BN) : rb;
         int j = rb;
         if constexpr (PF2) {
             if (n_fast - j >= 4) {
@@ -614,10 +640,14 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
     }
 
     const float l_tot = l_run + lane_xor32(l_run);
+    // CLS: what only the epilogue needs (output tensor, LSE, partial results) is read from the kernel's argument memory
+    // here instead of sitting in scalar registers through the loop, which has none to spare (the loop would re-read them
+    // from spill lanes in every step)
+    const AttnFwdParams& pe = CLS ? cold_params<AttnFwdParams>() : p;
     if (nparts > 1) {
         // ---- part of a split item: leave the unnormalised accumulators, m_ref and the row sum ----
         const int row = wave * 32 + li;
-        float* po = p.part_o + ((int64_t)part_id * ATTN_BM + row) * DPAD;
+        float* po = pe.part_o + ((int64_t)part_id * ATTN_BM + row) * DPAD;
 #pragma unroll
         for (int d = 0; d < NDB; ++d)
 #pragma unroll
@@ -625,7 +655,7 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
                 *reinterpret_cast<f32x4*>(po + d * 32 + g * 16 + e) =
                     f32x4{oacc[d][e], oacc[d][e + 1], oacc[d][e + 2], oacc[d][e + 3]};
         if (g == 0) {
-            float* pm = p.part_ml + ((int64_t)part_id * ATTN_BM + row) * 2;
+            float* pm = pe.part_ml + ((int64_t)part_id * ATTN_BM + row) * 2;
             pm[0] = m_ref;
             pm[1] = l_tot;
         }
@@ -633,13 +663,13 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
     }
     // ---- epilogue: normalise, write O and LSE ----
     const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-    T* op = static_cast<T*>(const_cast<void*>(p.o.ptr)) + b * p.o.sb + h * p.o.sh + (int64_t)q_row * p.o.sn;
+    T* op = static_cast<T*>(const_cast<void*>(pe.o.ptr)) + b * pe.o.sb + h * pe.o.sh + (int64_t)q_row * pe.o.sn;
     if (q_valid) {
 #pragma unroll
         for (int d = 0; d < NDB; ++d) {
             const int col = d * 32 + g * 16;
             if (vec) {
-                if (col < p.D) {
+                if (col < pe.D) {
                     Pack16 lo, hi;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
@@ -647,19 +677,19 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
                         hi.w[e] = pack2<T>(oacc[d][8 + 2 * e] * inv, oacc[d][8 + 2 * e + 1] * inv);
                     }
                     *reinterpret_cast<u32x4*>(op + col) = lo.v;
-                    if (col + 8 < p.D) *reinterpret_cast<u32x4*>(op + col + 8) = hi.v;
+                    if (col + 8 < pe.D) *reinterpret_cast<u32x4*>(op + col + 8) = hi.v;
                 }
             } else {
 #pragma unroll
                 for (int v = 0; v < 16; ++v)
-                    if (col + v < p.D) op[col + v] = static_cast<T>(oacc[d][v] * inv);
+                    if (col + v < pe.D) op[col + v] = static_cast<T>(oacc[d][v] * inv);
             }
         }
     }
-    if (g == 0 && q_row < p.Tq_rounded) {
+    if (g == 0 && q_row < pe.Tq_rounded) {
         // natural-log logsumexp; padding rows get a fixed value
         const float lse = q_valid ? (m_ref + __builtin_amdgcn_logf(l_tot)) * kLn2 : 0.f;
-        p.lse[(int64_t)bh * p.Tq_rounded + q_row] = lse;
+        pe.lse[(int64_t)bh * pe.Tq_rounded + q_row] = lse;
     }
 }
 
