@@ -16,10 +16,14 @@
  *   - return value 0 on success, negative rgd_status otherwise; rgd_last_error() returns a
  *     thread-local message for the last failure on the calling thread.
  *   - functions are re-entrant; the only state is the loaded code object and what rgd_init() caches.
- *   - stream capture: after rgd_init() has returned, every entry point makes no runtime call other than its
+ *   - stream capture: after rgd_init() has returned 0, every entry point makes no runtime call other than its
  *     kernel launches on `stream` (no allocation, copy, memset, attribute or device query, no
- *     hipGetLastError), so a sequence of calls may be recorded into a HIP graph.  The workspace queries
+ *     hipGetLastError unless a launch has failed), so a sequence of calls may be recorded into a HIP graph.
+ *     The one exception is rgd_rms_bwd_noalloc, which asks hipGetDevice for the current device on every call
+ *     (its scratch array has one address per GPU); hipGetDevice is allowed under capture.  The workspace queries
  *     (rgd_*_workspace, rgd_attn_seqlen_q_rounded) and rgd_version / rgd_last_error touch no stream at all.
+ *   - a launch that fails returns RGD_ERR_LAUNCH and is also cleared from the runtime's per-thread last error,
+ *     so the caller's next hipGetLastError reports the caller's own work.
  */
 #ifndef RGD_HIP_H
 #define RGD_HIP_H
@@ -66,10 +70,14 @@ typedef struct rgd_tensor4 {
 int         rgd_version(void);
 const char* rgd_last_error(void);
 
-/* One-time set-up: caches the compute-unit count of the current device and sets the LDS size attribute of
- * every attention kernel.  Thread-safe and idempotent; every entry point calls it on its own, so an explicit
- * call is only needed before the first entry point runs under stream capture (call it when the library is
- * loaded).  No counterpart in the reference (Triton configures kernels when it compiles them). */
+/* One-time set-up: caches the compute-unit count of the current device, sets the LDS size attribute of
+ * every attention kernel and resolves the scratch array of rgd_rms_bwd_noalloc on that device.  Thread-safe and
+ * idempotent; every entry point calls it on its own, so an explicit call is only needed before the first entry
+ * point runs under stream capture (call it when the library is loaded).  Returns RGD_ERR_LAUNCH while the process
+ * has no usable device (nothing is latched: a later call tries again), and the attention kernels' set-up status
+ * otherwise; a failure there is reported again by every attention entry point and leaves the row kernels
+ * (RMS, L2, head LayerNorm, RoPE) usable.  No counterpart in the reference (Triton configures kernels when it
+ * compiles them). */
 int rgd_init(void);
 
 /* ------------------------------------------------------------------------------------------
@@ -217,10 +225,16 @@ int64_t rgd_attn_seqlen_q_rounded(int64_t Tq);
 /* Tile classes of a bias matrix that the heads share (stride_h == 0), head dims up to 64.  Such a bias is usually a
  * mask (0 / -inf), and the reference streams it tile by tile for every head and in every kernel
  * (flash_attn/flash_attn_triton_cached.py:151-175, :430-470).  One pass over the matrix leaves two bits per tile of 32
- * queries x 64 keys (all +0, all -inf, anything else); rgd_attn_fwd and rgd_attn_bwd then run tiles that are all +0
- * like tiles without bias, leave all -inf tiles out and read the bias only for the others, with the same results bit
- * for bit.  Both calls make that pass themselves, into the end of their workspace, when bias_classes is NULL; a caller
- * that runs several calls on one bias (a forward and its backward) can make it once:
+ * queries x 64 keys (all +0; all -inf; every row equal to the tile's first row; anything else); rgd_attn_fwd and
+ * rgd_attn_bwd then run tiles that are all +0 like tiles without bias, leave all -inf tiles out and read the bias only
+ * for the others (one row of it where the rows are equal).  An all-+0 bias gives the results of a call without bias
+ * bit for bit.  In tiles that read the bias, the bias enters the logits before the q.k product is added instead of
+ * after it, and the dQ kernel adds do.v^T to -delta instead of subtracting delta afterwards: against a call that uses no
+ * classes, o, lse, dq, dk and dv agree to the last one or two bits of the tensor dtype, not bit for bit (a call is
+ * still reproducible bit for bit against itself).  Batch elements whose tiles are mostly of the last kind are run by
+ * the ordinary kernels, bit for bit as without classes.  Both calls make the pass themselves, into the end of their
+ * workspace, when bias_classes is NULL; a caller that runs several calls on one bias (a forward and its backward, or
+ * every layer of a model that shares one mask) can make it once:
  *   rgd_attn_bias_classes_bytes  size of the classes for this bias and shape; 0 when they would not be used
  *                                (bias not a matrix, not shared by the heads, rows not 16-byte aligned, D > 64, H < 2)
  *   rgd_attn_bias_classify       writes them (8-byte aligned buffer of that size), one kernel launch on `stream`
@@ -277,8 +291,10 @@ size_t rgd_attn_bwd_workspace(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int6
  * dS = P*(do v^T - delta)*scale, dk = dS^T q, dq = dS k.
  * dbias (NULL, or ptr NULL: none; the reference has none, flash_attn_triton_cached.py:1107) receives the bias
  * gradient P*(do v^T - delta) of every (query, key) pair in the bias dtype: a full (B,H,Tq,Tk) tensor by strides,
- * 16-byte aligned, rows at least Tk rounded up to 64 elements long (the padding is written too), which the caller
- * sums over the dimensions its bias broadcasts; with causal != 0 the caller clears it first (key tiles past the
+ * 16-byte aligned, rows at least Tk rounded up to 64 elements long, which the caller
+ * sums over the dimensions its bias broadcasts.  Columns up to Tk rounded up to the kernel's key tile (64 for head
+ * dims up to 64, 32 above) are written, the rest of a row is left as it was.  Every pair is rounded to the bias
+ * dtype before the caller's sum sees it.  With causal != 0 the caller clears it first (key tiles past the
  * diagonal are not visited).  Two-kernel form only.  dq, dk, dv are written
  * in the tensor dtype from fp32 accumulators, each exactly once; in a fixed order except for dq in the one-pass
  * form (see rgd_attn_bwd_mode).  bias_classes: NULL, or what rgd_attn_bias_classify wrote for this bias (used by the

@@ -122,7 +122,7 @@ constexpr AttnSplitModel kBwdSplit = {1.05f, 1.05f, 1.4f};
 
 int check_common(const char* name, int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, int dtype, int bias_kind,
                  int bias_dtype, const rgd_tensor4* bias) {
-    const int init_rc = rgd_ensure_init();
+    const int init_rc = rgd_attn_ready();
     if (init_rc != RGD_OK) return init_rc;
     RGD_REQUIRE(dtype == RGD_F16 || dtype == RGD_BF16, RGD_ERR_INVALID, "%s: Only support fp16 and bf16", name);
     RGD_REQUIRE(D >= 1 && D <= 128, RGD_ERR_INVALID, "%s: FlashAttention only support head dimensions up to 128", name);
@@ -165,7 +165,7 @@ size_t rgd_attn_bias_classes_bytes(int64_t B, int64_t H, int64_t Tq, int64_t Tk,
 int rgd_attn_bias_classify(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const rgd_tensor4* bias, int bias_kind,
                            int bias_dtype, void* classes, size_t classes_bytes, void* stream) {
     const char* name = "rgd_attn_bias_classify";
-    const int init_rc = rgd_ensure_init();
+    const int init_rc = rgd_attn_ready();
     if (init_rc != RGD_OK) return init_rc;
     const size_t need = rgd_attn_bias_classes_bytes(B, H, Tq, Tk, D, bias, bias_kind, bias_dtype);
     RGD_REQUIRE(need > 0, RGD_ERR_UNSUPPORTED, "%s: no tile classes for this bias and shape (rgd_attn_bias_classes_bytes is 0)", name);

@@ -22,14 +22,16 @@ void rgd_set_error(const char* fmt, ...);  // defined in api.hip
         }                                   \
     } while (0)
 
-// One-time set-up of the library (api.hip): compute-unit count, LDS size attributes of the attention kernels.
-// Every entry point calls it first; after the first call it is one atomic load, so in the steady state an
-// entry point makes no runtime call other than its kernel launches.
-int rgd_ensure_init();
-int rgd_num_cus();  // compute units of the device seen by the first call (256 when none could be queried)
+// One-time set-up of the library (api.hip): compute-unit count, LDS size attributes of the attention kernels, address
+// of the fixed scratch array.  Every entry point calls it first; once it has run on a process with a device it is one
+// atomic load, so in the steady state an entry point makes no runtime call other than its kernel launches.  A process
+// without a usable device latches nothing: the next call tries again.
+void rgd_ensure_init();
+int rgd_attn_ready();  // rgd_ensure_init, then the status of the attention kernels' set-up (error text set on failure)
+int rgd_num_cus();     // compute units of the device seen by the set-up (256 while none has been seen)
 
-// Kernel launch that returns its own error code (nothing is left behind for hipGetLastError).
-// Kernels take their parameter struct by value; a second scalar argument is allowed.
+// Kernel launch that returns its own error code.  Kernels take their parameter struct by value; a second scalar
+// argument is allowed.
 template <typename P>
 inline hipError_t rgd_launch(void (*kern)(P), dim3 grid, dim3 block, size_t lds, hipStream_t s, const P& p) {
     void* args[] = {const_cast<P*>(&p)};
@@ -40,7 +42,8 @@ inline hipError_t rgd_launch(void (*kern)(P, A), dim3 grid, dim3 block, size_t l
     void* args[] = {const_cast<P*>(&p), &a};
     return hipLaunchKernel(reinterpret_cast<const void*>(kern), grid, block, args, lds, s);
 }
-// hipError_t of a launch -> rgd_status, with the error text set
+// hipError_t of a launch -> rgd_status, with the error text set; a failure is also cleared from the runtime's
+// per-thread last error
 int rgd_launch_status(const char* what, hipError_t e);
 
 static inline bool rgd_dtype_ok(int d) { return d == RGD_F32 || d == RGD_F16 || d == RGD_BF16; }

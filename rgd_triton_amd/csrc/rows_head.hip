@@ -35,8 +35,7 @@ void fill_strides(int64_t (&dst)[3], const rgd_tensor4* t, bool token_inner) {
 int head_launch(const char* name, int mode, int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D,
                 const rgd_tensor4* xs[2], const rgd_tensor4* dys[2], const rgd_tensor4* ys[2], const RopeArgs* rope,
                 int dtype, float eps, int max_d, void* stream) {
-    const int init_rc = rgd_ensure_init();
-    if (init_rc != RGD_OK) return init_rc;
+    rgd_ensure_init();
     RGD_REQUIRE(rgd_dtype_ok(dtype), RGD_ERR_INVALID, "%s: Only support fp16, bf16, and fp32", name);
     RGD_REQUIRE(B >= 0 && H >= 0 && Tq >= 0 && Tk >= 0 && D >= 1, RGD_ERR_INVALID, "%s: negative shape", name);
     RGD_REQUIRE(D <= max_d, RGD_ERR_INVALID, "%s: Only supports head dimensions up to %d", name, max_d);

@@ -79,8 +79,7 @@ size_t wide_workspace(int64_t B, int64_t T1, int64_t C1, int64_t T2, int64_t C2)
 
 int wide_launch(const char* name, int op, bool bwd, int64_t B, const WideHalfArgs& a1, const WideHalfArgs& a2,
                 int dtype, float eps, void* workspace, size_t workspace_bytes, void* stream) {
-    const int init_rc = rgd_ensure_init();
-    if (init_rc != RGD_OK) return init_rc;
+    rgd_ensure_init();
     RGD_REQUIRE(rgd_dtype_ok(dtype), RGD_ERR_INVALID, "%s: Only support fp16, bf16, and fp32", name);
     RGD_REQUIRE(B >= 0 && B <= 65535, RGD_ERR_INVALID, "%s: batch %lld out of range", name, (long long)B);
     const WideHalfArgs* as[2] = {&a1, &a2};
@@ -323,8 +322,7 @@ int rgd_rms_bwd_noalloc(int64_t B, int64_t T, int64_t C, const rgd_tensor3* dy, 
                         const rgd_tensor3* w, const rgd_tensor3* dx, const rgd_tensor3* dw, int w_shared, int x_dtype,
                         int w_dtype, float eps, void* stream) {
     const char* name = "rgd_rms_bwd_noalloc";
-    const int init_rc = rgd_ensure_init();
-    if (init_rc != RGD_OK) return init_rc;
+    rgd_ensure_init();
     // the size rgd_rms_bwd_workspace asks a caller for must fit the fixed array
     RGD_REQUIRE(B >= 0 && T >= 0 && C >= 0, RGD_ERR_INVALID, "%s: negative shape", name);
     const size_t need = wide_workspace(B, T, C, 0, 0);
@@ -333,7 +331,7 @@ int rgd_rms_bwd_noalloc(int64_t B, int64_t T, int64_t C, const rgd_tensor3* dy, 
                 "rgd_rms_bwd with a workspace", name, (long long)B, (long long)T, (long long)C, need,
                 kNoAllocScratchBytes);
     void* ptr = nullptr;
-    const int rc = wide_noalloc_setup(&ptr);  // one atomic load once the device has been seen
+    const int rc = wide_noalloc_setup(&ptr);  // hipGetDevice and one atomic load once the device has been seen
     if (rc != RGD_OK) return rc;
     // every partial row the reduce kernel reads is written by this call's first kernel: nothing has to start at 0
     return wide_launch(name, WIDE_RMS, true, B, half(T, C, x, dy, dx, w, dw, w_dtype, w_shared), kNoHalf, x_dtype, eps,

@@ -559,11 +559,37 @@ def _bwd_mode(d):
     return _ATTN_BWD_MODES[_attn_bwd_mode]
 
 
+# bytes of the buffer that receives dS of every (query, key) pair when a bias gradient is asked for; a bias that
+# broadcasts over heads (or the batch) is served in chunks of heads (or batch elements) that fit it
+_DBIAS_CHUNK_BYTES = int(os.environ.get("RGD_DBIAS_CHUNK_MB", "256")) << 20
+
+
+def _attn_bwd_call(do, q, k, v, o, lse, dq, dk, dv, bias, causal, softmax_scale, mode, dfull, bias_classes):
+    """One rgd_attn_bwd launch sequence on (B, T, H, D) tensors or views of them; lse is contiguous (B, H, Tq_rounded)."""
+    batch, seqlen_q, nheads, d = q.shape
+    seqlen_k = k.shape[1]
+    lib = _hip.lib()
+    bdesc, bkind, bdtype = _bias_args(bias, q, seqlen_q, seqlen_k, batch, nheads)
+    ddesc = None
+    if dfull is not None:
+        ddesc = _hip.Tensor4(dfull.data_ptr(), dfull.stride(0), dfull.stride(1), dfull.stride(2))
+    nbytes = lib.rgd_attn_bwd_workspace(batch, nheads, seqlen_q, seqlen_k, d, mode)
+    ws = _hip.workspace(q.device, nbytes)
+    _hip.check(lib.rgd_attn_bwd(batch, nheads, seqlen_q, seqlen_k, d, t4(do, False), t4(q, False), t4(k, False),
+                                t4(v, False), t4(o, False), ctypes.c_void_p(lse.data_ptr()), bdesc, bkind, bdtype,
+                                t4(dq, False), t4(dk, False), t4(dv, False), ddesc, _hip.dtype_code(q.dtype),
+                                int(bool(causal)), float(softmax_scale), mode,
+                                bias_classes.data_ptr() if bias_classes is not None else None, ws.data_ptr(), nbytes,
+                                _hip.stream_ptr(q.device)), "rgd_attn_bwd")
+
+
 def _flash_attn_backward(do, q, k, v, o, lse, dq, dk, dv, bias=None, causal=False, softmax_scale=None,
                          kernel_cache=None, bias_grad=False, bias_classes=None):
     """Returns None, or with bias_grad the gradient of `bias` in its own shape and dtype (beyond the reference, which
-    refuses it, flash_attn_triton_cached.py:1107): the dQ kernel leaves dS of every (query, key) pair in a full
-    (B, H, Tq, Tk) buffer and the dimensions the bias broadcasts are summed here in fp32."""
+    refuses it, flash_attn_triton_cached.py:1107): the dQ kernel leaves dS of every (query, key) pair, rounded to the
+    bias dtype, in a (B, H, Tq, Tk) buffer and the dimensions the bias broadcasts are summed here in fp32.  A bias
+    that broadcasts over the heads (else: over the batch) is served in chunks of heads (batch elements), so that the
+    buffer stays within RGD_DBIAS_CHUNK_MB (256) MiB where one head (batch element) fits that."""
     if do.stride(-1) != 1:
         do = do.contiguous()
     batch, seqlen_q, nheads, d = q.shape
@@ -577,30 +603,46 @@ def _flash_attn_backward(do, q, k, v, o, lse, dq, dk, dv, bias=None, causal=Fals
         assert dq.stride(-1) == dk.stride(-1) == dv.stride(-1) == 1
     _seen(kernel_cache, "bwd_odot", _sig(o, do))
     softmax_scale = softmax_scale or 1.0 / math.sqrt(d)
-    bdesc, bkind, bdtype = _bias_args(bias, q, seqlen_q, seqlen_k, batch, nheads)
-    mode = _bwd_mode(d)
-    dfull, ddesc = None, None
-    if bias_grad:
-        mode = _hip.ATTN_BWD_TWO_KERNEL  # the dQ kernel writes the bias gradient
-        tk_pad = (seqlen_k + 63) // 64 * 64  # rows of whole 64-key tiles
-        alloc = torch.zeros if causal else torch.empty  # key tiles past the causal diagonal are not visited
-        dfull = alloc((batch, nheads, seqlen_q, tk_pad), dtype=bias.dtype, device=q.device)
-        ddesc = _hip.Tensor4(dfull.data_ptr(), dfull.stride(0), dfull.stride(1), dfull.stride(2))
-    nbytes = lib.rgd_attn_bwd_workspace(batch, nheads, seqlen_q, seqlen_k, d, mode)
-    ws = _hip.workspace(q.device, nbytes)
-    _hip.check(lib.rgd_attn_bwd(batch, nheads, seqlen_q, seqlen_k, d, t4(do, False), t4(q, False), t4(k, False),
-                                t4(v, False), t4(o, False), ctypes.c_void_p(lse.data_ptr()), bdesc, bkind, bdtype,
-                                t4(dq, False), t4(dk, False), t4(dv, False), ddesc, _hip.dtype_code(q.dtype),
-                                int(bool(causal)), float(softmax_scale), mode,
-                                bias_classes.data_ptr() if bias_classes is not None else None, ws.data_ptr(), nbytes,
-                                _hip.stream_ptr(q.device)), "rgd_attn_bwd")
     if not bias_grad:
+        _attn_bwd_call(do, q, k, v, o, lse, dq, dk, dv, bias, causal, softmax_scale, _bwd_mode(d), None, bias_classes)
         return None
-    dfull = dfull[..., :seqlen_k]
-    dims = [i for i in range(4) if bias.shape[i] == 1 and dfull.shape[i] != 1]
-    if dims:
-        return dfull.sum(dim=dims, keepdim=True, dtype=torch.float32).to(bias.dtype)
-    return dfull.contiguous()
+
+    mode = _hip.ATTN_BWD_TWO_KERNEL  # the dQ kernel writes the bias gradient
+    tk_pad = (seqlen_k + 63) // 64 * 64  # rows of whole 64-key tiles
+    alloc = torch.zeros if causal else torch.empty  # key tiles past the causal diagonal are not visited
+    over_heads = bias.shape[1] == 1 and nheads > 1
+    over_batch = bias.shape[0] == 1 and batch > 1
+    pair_bytes = seqlen_q * tk_pad * bias.element_size()
+    hc, bc = nheads, batch
+    if over_heads:
+        hc = max(1, min(nheads, _DBIAS_CHUNK_BYTES // max(1, batch * pair_bytes)))
+    elif over_batch:
+        bc = max(1, min(batch, _DBIAS_CHUNK_BYTES // max(1, nheads * pair_bytes)))
+    if hc == nheads and bc == batch:
+        dfull = alloc((batch, nheads, seqlen_q, tk_pad), dtype=bias.dtype, device=q.device)
+        _attn_bwd_call(do, q, k, v, o, lse, dq, dk, dv, bias, causal, softmax_scale, mode, dfull, None)
+        dfull = dfull[..., :seqlen_k]
+        dims = [i for i in range(4) if bias.shape[i] == 1 and dfull.shape[i] != 1]
+        if dims:
+            return dfull.sum(dim=dims, keepdim=True, dtype=torch.float32).to(bias.dtype)
+        return dfull.contiguous()
+
+    acc = torch.zeros(bias.shape, dtype=torch.float32, device=q.device)
+    buf = alloc((bc, hc, seqlen_q, tk_pad), dtype=bias.dtype, device=q.device)
+    for b0 in range(0, batch, bc):
+        for h0 in range(0, nheads, hc):
+            bs, hs = slice(b0, min(batch, b0 + bc)), slice(h0, min(nheads, h0 + hc))
+            part = buf[: bs.stop - bs.start, : hs.stop - hs.start]
+            if causal and (b0 or h0):
+                part.zero_()
+            bias_part = bias[bs if bias.shape[0] > 1 else slice(None), hs if bias.shape[1] > 1 else slice(None)]
+            _attn_bwd_call(do[bs, :, hs], q[bs, :, hs], k[bs, :, hs], v[bs, :, hs], o[bs, :, hs], lse[bs, hs].contiguous(),
+                           dq[bs, :, hs], dk[bs, :, hs], dv[bs, :, hs], bias_part, causal, softmax_scale, mode, part, None)
+            got = part[..., :seqlen_k]
+            dims = [i for i in range(4) if bias.shape[i] == 1 and got.shape[i] != 1]
+            got = got.sum(dim=dims, keepdim=True, dtype=torch.float32) if dims else got.float()
+            acc[bs if bias.shape[0] > 1 else slice(None), hs if bias.shape[1] > 1 else slice(None)] += got
+    return acc.to(bias.dtype)
 
 
 class FlashAttnFunc(torch.autograd.Function):

@@ -670,6 +670,33 @@ def test_flash_attn_bias_gradient(d, Tq, Tk, bias_type, causal, bias_dtype, dtyp
     assert maxdiff(db, ref) <= allowed, f"dbias error {maxdiff(db, ref)} (allowed {allowed}, scale {scale}, {terms} terms)"
 
 
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("bias_type", ["static", "batch", "head", "vector"])
+def test_flash_attn_bias_gradient_in_chunks(bias_type, causal, monkeypatch):
+    """A bias that broadcasts over heads (else: over the batch) has its gradient formed in chunks of heads (batch
+    elements) that fit a bounded buffer.  With the bound forced down to one head / one batch element per chunk, dq, dk
+    and dv are the unchunked ones bit for bit, and the bias gradient differs only in how its fp32 sum is grouped."""
+    from rgd_triton_amd import flash_attn_func, functional
+
+    g = gen(15)
+    B, H, Tq, Tk, d, dtype = 3, 5, 150, 200, 64, torch.bfloat16
+    q, k, v, do = (randn(g, B, T, H, d, dtype=dtype).cuda() for T in (Tq, Tk, Tk, Tq))
+    bias = make_bias(g, bias_type, B, H, Tq, Tk, dtype).cuda().requires_grad_(True)
+    qg, kg, vg = (t.requires_grad_(True) for t in (q, k, v))
+
+    def grads():
+        return torch.autograd.grad(flash_attn_func(qg, kg, vg, bias, causal), (qg, kg, vg, bias), do)
+
+    whole = grads()
+    monkeypatch.setattr(functional, "_DBIAS_CHUNK_BYTES", 1)
+    chunked = grads()
+    for a, b in zip(whole[:3], chunked[:3]):
+        assert torch.equal(a, b)
+    assert chunked[3].shape == bias.shape and chunked[3].dtype == bias.dtype
+    scale = whole[3].float().abs().max().item()
+    assert maxdiff(chunked[3], whole[3].cpu()) <= 2 * half_ulp(dtype) * scale
+
+
 @pytest.mark.parametrize("dtype", HALF)
 @pytest.mark.parametrize("B,H,T,d,with_bias,mode", [(1, 2, 2048, 64, False, 1), (1, 3, 1536, 128, True, 1), (2, 5, 1100, 32, True, 1),
                                                     (1, 2, 2048, 64, False, 2), (2, 5, 1100, 32, True, 2)])

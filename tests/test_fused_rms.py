@@ -105,11 +105,11 @@ RACE_PAIRS = [(1, 239), (239, 1), (3, 799), (799, 3), (1024, 128), (97, 97), (12
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("unique_bw", [True, False])
-@pytest.mark.parametrize("C,dfactor", [(63, -0.75), (384, 0.6), (1023, 1.0)])
+@pytest.mark.parametrize("C,dfactor", [(63, -0.75), (122, 0.2), (384, 0.6), (384, -0.3), (740, -0.3), (1023, 1.0)])
 @pytest.mark.parametrize("T1,T2", RACE_PAIRS)
 def test_fused_rms_norm_race_condition(T1, T2, C, dfactor, unique_bw, dtype):
-    """The reference's race test (tests/test_fused_rms.py:331-): batch 60, its 14 length pairs, 250 repeats, on three
-    of its nine widths and two of its five width ratios; every output and gradient must reproduce bit for bit."""
+    """The reference's race test (tests/test_fused_rms.py:331-): batch 60, its 14 length pairs, 250 repeats, on five
+    of its nine widths (one of them with two ratios) and all five of its width ratios; every output and gradient must reproduce bit for bit."""
     from rgd_triton_amd import triton_fused_rms_func_fn
 
     g = gpu_gen(13)

@@ -235,11 +235,11 @@ def test_head_ln_race_condition(Tq, Tk, D, heads_second, dtype):
 @pytest.mark.parametrize("which", ["rope", "ln_rope"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 @pytest.mark.parametrize("heads_second", [True, False])
-@pytest.mark.parametrize("D,R", [(64, 32), (128, 96)])
+@pytest.mark.parametrize("D,R", [(32, 32), (64, 32), (128, 96), (128, 128)])
 @pytest.mark.parametrize("Tq,Tk", RACE_PAIRS)
 def test_rope_race_condition(Tq, Tk, D, R, heads_second, dtype, which):
     """The race tests of tests/test_head_rope.py and tests/test_fused_ln_rope.py: batch 60, their 14 length pairs, 250
-    repeats, on two of their (head dim, rotary dim) combinations; cutoffs inside both sequences."""
+    repeats, on four of their seven (head dim, rotary dim) combinations; cutoffs inside both sequences."""
     from rgd_triton_amd import triton_fused_ln_rope_fn, triton_rope_fn
 
     g = gpu_gen(6)

@@ -121,12 +121,13 @@ FUSED_RACE_PAIRS = [(1, 239), (239, 1), (3, 799), (799, 3), (1024, 128), (97, 97
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("d,dfactor", [(32, -0.75), (97, -0.3), (257, 0.2), (510, 0.6), (1023, 1.0)])
+@pytest.mark.parametrize("d,dfactor", [(32, -0.75), (63, 0.6), (97, -0.3), (122, 1.0), (257, 0.2), (257, -0.75), (384, -0.3),
+                                       (510, 0.6), (740, 0.2), (1023, 1.0)])
 @pytest.mark.parametrize("Tq,Tk", FUSED_RACE_PAIRS)
 def test_fused_l2_norm_race_condition(Tq, Tk, d, dfactor, dtype):
     """The race test of tests/test_fused_l2normalize.py:283-354: batch 60, its 14 (Tq, Tk) pairs, 250 repeats of forward
-    + backward; the widths follow its rule (dfactor < 0 narrows the first input, else the second).  One (d, dfactor)
-    pairing per width instead of its full 9 x 5 grid."""
+    + backward; the widths follow its rule (dfactor < 0 narrows the first input, else the second).  Every one of its
+    nine widths with one ratio (one width with two) instead of its full 9 x 5 grid."""
     from rgd_triton_amd import triton_fused_norm_func_fn
 
     CQ, CK = (int(-dfactor * d), d) if dfactor < 0 else (d, int(dfactor * d))

@@ -30,10 +30,14 @@ def _both(lib, hip, B, T, C, dtype, wdtype, shared, seed):
             rc = lib.rgd_rms_bwd(B, T, C, t3(dyg), t3(xg), t3(wg, wsb), t3(dx), t3(dw, dwsb), int(shared), code, wcode,
                                  1e-6, ws.data_ptr(), n, st)
         else:
-            before = torch.cuda.memory_allocated()
+            # neither torch's allocator nor the device itself (an allocation made behind torch's back) gives up memory
+            torch.cuda.synchronize()
+            before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
             rc = lib.rgd_rms_bwd_noalloc(B, T, C, t3(dyg), t3(xg), t3(wg, wsb), t3(dx), t3(dw, dwsb), int(shared), code,
                                          wcode, 1e-6, st)
+            torch.cuda.synchronize()
             assert torch.cuda.memory_allocated() == before
+            assert torch.cuda.mem_get_info()[0] >= free_before
         assert rc == 0, lib.rgd_last_error()
         torch.cuda.synchronize()
         out[which] = (dx, dw)
