@@ -57,8 +57,6 @@ int64_t bwd_rows32(int64_t Tq) { return (Tq + BWD_BM - 1) / BWD_BM * (BWD_BM / 3
 size_t bwd_ranges_bytes(int64_t B, int64_t H, int64_t Tq, int dpad) {
     return dpad > 64 ? (size_t)(B * H * bwd_rows32(Tq)) * 2 * sizeof(int) : 0;
 }
-// dK/dV launches with tile classes: one byte per (batch, key block), see AttnBwdParams::cls_served
-size_t bwd_served_bytes(int64_t B, int64_t Tk) { return ((size_t)(B * ((Tk + BWD_BM - 1) / BWD_BM)) + 15) & ~(size_t)15; }
 size_t bwd_delta_bytes(int64_t B, int64_t H, int64_t Tq) { return (size_t)(B * H * rgd_attn_seqlen_q_rounded(Tq)) * sizeof(float); }
 // one-pass form: fp32 dq_accum (B, H, Tq_rounded, DPAD) behind delta
 size_t bwd_accum_bytes(int64_t B, int64_t H, int64_t Tq, int dpad) { return bwd_delta_bytes(B, H, Tq) * (size_t)dpad; }
@@ -81,13 +79,8 @@ bool cls_eligible(int64_t H, int64_t Tq, int64_t Tk, int64_t D, const rgd_tensor
     return cls_nwords(Tk) <= CLS_MAX_WORDS && cls_nrow32(Tq) <= CLS_MAX_ROWS;
 }
 int64_t cls_batches(int64_t B, const rgd_tensor4* bias) { return bias->stride_b == 0 ? 1 : B; }
-BiasClasses cls_desc(const void* words, int64_t B, int64_t Tq, int64_t Tk, const rgd_tensor4* bias) {
-    BiasClasses c;
-    c.words = static_cast<const uint64_t*>(words);
-    c.nwords = cls_nwords(Tk);
-    c.nrow32 = cls_nrow32(Tq);
-    c.sb = cls_batches(B, bias) == 1 ? 0 : (int64_t)c.nrow32 * c.nwords;
-    return c;
+BiasClasses cls_desc(const void* buffer, int64_t B, int64_t Tq, int64_t Tk, const rgd_tensor4* bias) {
+    return cls_layout(buffer, cls_batches(B, bias), Tq, Tk);
 }
 // The classes a call works with: the caller's (bias_classes), or written here into the end of the workspace when it has
 // room for them behind `fixed_bytes`; *room is what is left of the workspace in front of them.  Null: none.
@@ -272,7 +265,7 @@ size_t rgd_attn_bwd_workspace(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int6
     const int dpad = attn_dpad(D < 1 ? 1 : D);
     const bool accum = mode != RGD_ATTN_BWD_TWO_KERNEL && D <= 64 && (mode == RGD_ATTN_BWD_ONE_PASS || RGD_ATTN_BWD_AUTO_ONE_PASS);
     const size_t cls = (D <= 64 && B > 0 && Tq > 0 && Tk > 0 && cls_nwords(Tk) <= CLS_MAX_WORDS && cls_nrow32(Tq) <= CLS_MAX_ROWS)
-                           ? cls_bytes(B, Tq, Tk) + 32 + bwd_served_bytes(B, Tk)
+                           ? cls_bytes(B, Tq, Tk) + 32
                            : 0;
     return bwd_delta_bytes(B, H, Tq) + (accum ? bwd_accum_bytes(B, H, Tq, dpad) : 0) +
            (size_t)2 * rgd_num_cus() * bwd_blocks_per_cu(dpad) * bwd_part_bytes(dpad, 2) + bwd_ranges_bytes(B, H, Tq, dpad) + 16 + cls;
@@ -341,19 +334,12 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
     // tile classes of a head-shared bias (two-kernel form, no bias gradient): the caller's, or written into the end of
     // the workspace
     const void* cls = nullptr;
-    uint8_t* cls_served = nullptr;
-    const size_t served_bytes = bwd_served_bytes(B, Tk);
-    if (!one_pass && !want_dbias && Tq > 0 && Tk > 0 && softmax_scale > 0.f && workspace_bytes >= fixed_bytes + served_bytes) {
-        // the bytes in which the two dK/dV launches agree on who serves a key block sit behind delta
+    if (!one_pass && !want_dbias && Tq > 0 && Tk > 0 && softmax_scale > 0.f) {
         size_t tail = workspace_bytes;
         cls = cls_for_call(name, B, H, Tq, Tk, D, bias, bias_kind, bias_dtype, bias_classes, workspace, workspace_bytes,
-                           fixed_bytes + served_bytes, &tail, s, &rc);
+                           fixed_bytes, &tail, s, &rc);
         if (rc != RGD_OK) return rc;
-        if (cls) {
-            cls_served = reinterpret_cast<uint8_t*>(static_cast<char*>(workspace) + fixed_bytes);
-            part_base = reinterpret_cast<float*>(static_cast<char*>(workspace) + fixed_bytes + served_bytes);
-            part_room = tail - fixed_bytes - served_bytes;
-        }
+        if (cls) part_room = tail - fixed_bytes;
     }
 
     AttnBwdParams p;
@@ -393,7 +379,6 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
                      (p.bias.sn % per16) == 0;
     }
     if (cls) p.cls = cls_desc(cls, B, Tq, Tk, bias);
-    p.cls_served = cls_served;
     if (one_pass) {
         p.dq_accum = reinterpret_cast<float*>(static_cast<char*>(workspace) + delta_bytes);
         if (Tq > 0) {  // delta, and dq_accum = 0

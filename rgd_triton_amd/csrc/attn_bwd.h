@@ -67,10 +67,7 @@ struct AttnBwdParams {
     // workgroups this launch serves when the classes came with two launches (see cls_batch_dense): 0 all, 1 only batch
     // elements whose bias is mostly ZERO / NEG tiles, 2 only the others.
     BiasClasses cls;
-    int cls_take;
-    // dK/dV launches with classes: one byte per (batch, key block), written by the CLS launch (1: a key mask block, served
-    // there) and read by the ordinary launch behind it, which then need not look at the bias to know what is left for it
-    uint8_t* cls_served;
+    int cls_take;  // dK/dV launches: 1 only the "key mask" blocks of the classes' summary, 2 only the others
 };
 
 // block id -> (logical item, part, number of parts, part id)
@@ -204,7 +201,7 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
     if constexpr (HAS_BIAS && !DBIAS && DPAD <= 64) {
         // classes came with two launches over the same grid: this one serves the batch elements of its kind
         if (p.cls_take != 0) {
-            if (cls_batch_dense(p.cls, b, (p.Tk + CLS_KEYS - 1) / CLS_KEYS, lane) != (p.cls_take == 2)) return;
+            if (cls_batch_dense(p.cls, b) != (p.cls_take == 2)) return;
         }
     }
     const int q_row = qb * BWD_BM + wave * 32 + li;
@@ -739,14 +736,13 @@ template <typename TB> struct BiasColumn {
 // CLS: the bias comes with tile classes (attn_classes.h).  The kernel is the one without bias (same loop, two 32-row
 // sub-tiles per step); it serves the key blocks that a padding mask leaves as "key mask" blocks (cls_key_mask_block): their
 // hidden keys are treated like keys that do not exist.  Every other key block leaves at once and runs in the ordinary biased
-// kernel, which is launched over the same grid behind this one (cls_take == 2) and leaves the key mask blocks alone.
+// kernel, which is launched over the same grid (cls_take == 2) and leaves the key mask blocks alone.
 template <typename T, int DPAD, int BIAS, bool FUSED = false, bool CLS = false>
 __global__ __launch_bounds__(BWD_THREADS, dkv_occupancy(DPAD, CLS ? BIAS_OFF : BIAS, FUSED)) void attn_bwd_dkv_kernel(const AttnBwdParams p) {
     constexpr bool HAS_BIAS = BIAS != BIAS_OFF;
     static_assert(!CLS || (HAS_BIAS && !FUSED && DPAD <= 64), "tile classes: head dims up to 64, with a bias, two-kernel form");
     constexpr bool BIAS_AHEAD = HAS_BIAS && !CLS;  // bias registers fetched one step ahead of use
     typedef typename BiasElem<T, BIAS>::type TB;
-    typedef TB TB_;
     typedef Mfma<T> MM;
     constexpr int NSUB = dkv_nsub(DPAD, CLS ? BIAS_OFF : BIAS, FUSED);
     typedef DkvSmem<DPAD, NSUB, FUSED> SM;
@@ -781,20 +777,16 @@ __global__ __launch_bounds__(BWD_THREADS, dkv_occupancy(DPAD, CLS ? BIAS_OFF : B
     if constexpr (HAS_BIAS && !FUSED && DPAD <= 64) {
         // classes came with two launches over the same grid: key mask blocks run here when CLS, all others when not
         if (p.cls_take != 0) {
-            uint8_t* served = p.cls_served + (int64_t)b * p.nblk + kblk;
+            static_assert(BWD_BM == CLS_KEY_BLOCK, "one summary entry per workgroup of this kernel");
+            const uint32_t* entry = cls_key_block(p.cls, b, kblk);
+            const uint32_t flags = entry[4];
+            if (((flags & CLS_KB_PURE) != 0) != CLS) return;
             if constexpr (CLS) {
-                const TB_* key_col = static_cast<const TB_*>(p.bias.ptr) + b * p.bias.sb + h * p.bias.sh + k_ld;
-                bool hidden, any_hidden, all_hidden;
-                const bool pure = cls_key_mask_block<TB_>(p.cls, key_col, p.bias.sn, b, kblk * (BWD_BM / CLS_KEYS),
-                                                          min((p.Tq + CLS_ROWS - 1) / CLS_ROWS, p.cls.nrow32), p.Tq, lane, tid,
-                                                          reinterpret_cast<int*>(smem_raw), hidden, any_hidden, all_hidden);
-                if (tid == 0) *served = pure ? 1 : 0;  // every head of the batch element writes the same value
-                if (!pure) return;
+                const int kl = wave * 32 + li;  // this lane's key within the block
+                const bool hidden = ((entry[kl >> 5] >> (kl & 31)) & 1u) != 0;
                 k_valid = k_valid && !hidden;
-                no_key_hidden = !any_hidden;
-                all_keys_hidden = all_hidden;
-            } else {
-                if (*served != 0) return;
+                no_key_hidden = (flags & CLS_KB_ANY_HIDDEN) == 0;
+                all_keys_hidden = (flags & CLS_KB_ALL_HIDDEN) != 0;
             }
         }
     }

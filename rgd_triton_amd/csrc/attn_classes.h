@@ -25,17 +25,47 @@ constexpr int CLS_TILES_PER_WORD = 32;
 constexpr int CLS_MAX_WORDS = 64;      // up to 2048 key tiles (131072 keys): one byte each in LDS
 constexpr int CLS_MAX_ROWS = 4096;     // up to 2048 steps of 64 query rows (131072 rows): one byte each in LDS
 
+constexpr int CLS_KEY_BLOCK = 128;     // keys per workgroup of the dK/dV kernel at head dims up to 64
+constexpr int CLS_INFO_HEAD = 4;       // 32-bit words of a batch element's summary in front of its key block entries
+constexpr int CLS_INFO_ENTRY = 8;      // 32-bit words per key block entry
+
+// Behind the map lies a summary per batch element, written by a second launch (attn_bias_summary_kernel), so that no
+// workgroup of the attention kernels has to derive it again:
+//     info[b * info_sb + 0]                             1: most tiles are MIXED, the ordinary biased kernels serve b
+//     info[b * info_sb + CLS_INFO_HEAD + kb * 8 + 0..3]  key block kb (128 keys): bit k set = key k is hidden from every query
+//     info[b * info_sb + CLS_INFO_HEAD + kb * 8 + 4]     bit 0: "key mask" block (see attn_bias_summary_kernel), bit 1: some key
+//                                                       of it is hidden, bit 2: every key of it is
 struct BiasClasses {
     const uint64_t* words;  // null: no classes for this call
     int nwords;             // words per row of 32 query rows
     int nrow32;             // rows of the map per batch element
     int64_t sb;             // words between batch elements (0: one map for every batch element)
+    const uint32_t* info;   // summaries, behind the words
+    int64_t info_sb;        // 32-bit words between the summaries of two batch elements (0: one for all)
 };
+enum { CLS_KB_PURE = 1, CLS_KB_ANY_HIDDEN = 2, CLS_KB_ALL_HIDDEN = 4 };
 
 // host: shape of the map for a (Tq, Tk) bias
 inline int cls_nwords(int64_t Tk) { return (int)(((Tk + CLS_KEYS - 1) / CLS_KEYS + CLS_TILES_PER_WORD - 1) / CLS_TILES_PER_WORD); }
 inline int cls_nrow32(int64_t Tq) { return (int)((Tq + 127) / 128 * 4); }
-inline size_t cls_bytes(int64_t nb, int64_t Tq, int64_t Tk) { return (size_t)nb * cls_nrow32(Tq) * cls_nwords(Tk) * sizeof(uint64_t); }
+inline int cls_nkb(int64_t Tk) { return (int)((Tk + CLS_KEY_BLOCK - 1) / CLS_KEY_BLOCK); }
+inline size_t cls_words_bytes(int64_t nb, int64_t Tq, int64_t Tk) { return (size_t)nb * cls_nrow32(Tq) * cls_nwords(Tk) * sizeof(uint64_t); }
+inline int64_t cls_info_words(int64_t Tk) { return CLS_INFO_HEAD + (int64_t)cls_nkb(Tk) * CLS_INFO_ENTRY; }
+inline size_t cls_bytes(int64_t nb, int64_t Tq, int64_t Tk) {
+    return cls_words_bytes(nb, Tq, Tk) + (size_t)nb * cls_info_words(Tk) * sizeof(uint32_t);
+}
+
+// host: the parts of a classes buffer written for nb batch elements (nb = 1: one map that every batch element uses)
+inline BiasClasses cls_layout(const void* buffer, int64_t nb, int64_t Tq, int64_t Tk) {
+    BiasClasses c;
+    c.words = static_cast<const uint64_t*>(buffer);
+    c.nwords = cls_nwords(Tk);
+    c.nrow32 = cls_nrow32(Tq);
+    c.sb = nb == 1 ? 0 : (int64_t)c.nrow32 * c.nwords;
+    c.info = reinterpret_cast<const uint32_t*>(static_cast<const char*>(buffer) + cls_words_bytes(nb, Tq, Tk));
+    c.info_sb = nb == 1 ? 0 : cls_info_words(Tk);
+    return c;
+}
 
 constexpr int CLS_LDS_BYTES = 2048;  // forward and dQ kernel: one byte per key tile
 
@@ -57,59 +87,6 @@ __device__ __forceinline__ void cls_tiles_to_lds(const BiasClasses& c, int b, in
     }
     __syncthreads();
 }
-// dK/dV kernel.  A workgroup owns 128 keys and walks the query rows; what a padding mask does to it does not change along
-// the way: a key is hidden from every query or from none.  Such a key block is a "key mask" block: no tile of its two key
-// tiles is MIXED, and for each of its keys the bias is +0 in every row or -inf in every row.  It then runs the loop of the
-// kernel without bias, with its hidden keys treated like keys that do not exist (their probabilities are 0), and is left
-// alone by the ordinary biased kernel that is launched behind it; every other key block leaves at once and is served by
-// that kernel.  Both kernels call this function, so both decide alike.
-//   key_col: &bias[b, h, 0, this lane's key] (an existing key); rows32: rows of the map that hold query rows.
-//   slot: two ints in LDS nothing else uses.  Returns (the same in every lane of the workgroup) whether the block is a key
-//   mask block; hidden: this lane's key is hidden; any_hidden / all_hidden: some / every key of the workgroup is.
-template <typename TB>
-__device__ __forceinline__ bool cls_key_mask_block(const BiasClasses& c, const TB* __restrict__ key_col, int64_t sn, int b, int tile0, int rows32,
-                                                   int Tq, int lane, int tid, int* slot, bool& hidden, bool& any_hidden, bool& all_hidden) {
-    typedef typename std::conditional<sizeof(TB) == 2, uint16_t, uint32_t>::type Bits;
-    constexpr Bits NEG = (Bits)(NegInfBits<TB>::value & (sizeof(TB) == 2 ? 0xFFFFu : 0xFFFFFFFFu));
-    // no MIXED tile in the two columns of the map: every thread looks at some of the rows
-    bool ok = true;
-    for (int r = tid; r < rows32; r += 256) {
-        const uint32_t v = (uint32_t)(c.words[b * c.sb + (int64_t)r * c.nwords + (tile0 >> 5)] >> (2 * (tile0 & 31)));
-        ok = ok && (v & 3u) != CLS_MIXED && ((v >> 2) & 3u) != CLS_MIXED;
-    }
-    // every 32 rows of such a column are the same row: the first one stands for them
-    Bits all_and = (Bits)~(Bits)0, all_or = 0;
-    for (int r0 = 0; r0 < rows32; r0 += 8) {
-        Bits v[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = __builtin_bit_cast(Bits, key_col[(int64_t)min((r0 + i) * CLS_ROWS, Tq - 1) * sn]);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            all_and &= v[i];
-            all_or |= v[i];
-        }
-    }
-    hidden = all_and == NEG && all_or == NEG;
-    const bool plain = all_or == 0;
-    ok = ok && (hidden || plain);
-    if (tid == 0) {
-        slot[0] = 1;  // all ok
-        slot[1] = 0;  // bit 0: some key hidden, bit 1: some key not hidden
-    }
-    __syncthreads();
-    const bool wave_bad = __builtin_amdgcn_ballot_w64(!ok) != 0;
-    const int wave_bits = (__builtin_amdgcn_ballot_w64(hidden) != 0 ? 1 : 0) | (__builtin_amdgcn_ballot_w64(!hidden) != 0 ? 2 : 0);
-    if (lane == 0) {
-        if (wave_bad) slot[0] = 0;
-        atomicOr(&slot[1], wave_bits);
-    }
-    __syncthreads();
-    const bool pure = slot[0] != 0;
-    any_hidden = (slot[1] & 1) != 0;
-    all_hidden = (slot[1] & 2) == 0;
-    __syncthreads();  // the slot's memory is free again
-    return pure;
-}
 // class of tile / step j, the same value in every lane (a scalar for the compiler)
 __device__ __forceinline__ int cls_lds_at(const uint8_t* lds, int j) { return __builtin_amdgcn_readfirstlane((int)lds[j]); }
 
@@ -121,23 +98,103 @@ __device__ __forceinline__ int cls_count_mixed(uint64_t w, int n) {
 }
 
 // Which kernels serve a batch element.  A bias with classes is launched twice over the same grid: the CLS variant of
-// the kernel (laid out like the kernel without bias; reads the bias only in the runs of MIXED tiles, at the start of each
-// step) and the ordinary biased kernel (bias fetched a tile ahead in every step).  Every workgroup of both launches asks
-// this function about its batch element and leaves at once if the other launch serves it: true (ordinary kernel) when more
-// than half of a fixed sample of the map (64 of its words, evenly spaced) is MIXED, i.e. the bias is a dense one.  The
-// same answer in every lane of every workgroup that asks: all items of a batch element run in one launch.
-__device__ __forceinline__ bool cls_batch_dense(const BiasClasses& c, int b, int ntiles, int lane) {
-    const int total = c.nrow32 * c.nwords;
-    const int i = (int)((int64_t)lane * total / 64);  // 64 words, evenly spaced (all of them when the map has at most 64)
-    const int w = i % c.nwords;
-    const int n = min(32, ntiles - 32 * w);  // tiles of that word that exist
-    int mixed = cls_count_mixed(c.words[b * c.sb + i], n), seen = n;
+// the kernel (laid out like the kernel without bias; reads the bias only for the tiles that are not ZERO, at the start of
+// their step) and the ordinary biased kernel (bias fetched a tile ahead in every step).  Every workgroup of both launches
+// reads this flag of its batch element and leaves at once if the other launch serves it.
+__device__ __forceinline__ bool cls_batch_dense(const BiasClasses& c, int b) {
+    return __builtin_amdgcn_readfirstlane((int)c.info[b * c.info_sb]) != 0;
+}
+// dK/dV kernel: the entry of key block kb (uniform address: the compiler reads it through the scalar cache)
+__device__ __forceinline__ const uint32_t* cls_key_block(const BiasClasses& c, int b, int kb) {
+    return c.info + b * c.info_sb + CLS_INFO_HEAD + (int64_t)kb * CLS_INFO_ENTRY;
+}
+
+// Second launch of the classification, grid (key blocks + 1, batch elements), 256 threads.
+//
+// Workgroup kb < nkb writes the entry of key block kb for the dK/dV kernel.  A workgroup of that kernel owns 128 keys and
+// walks the query rows; what a padding mask does to it does not change along the way: a key is hidden from every query
+// or from none.  Such a key block is a "key mask" block: no tile of its two key tiles is MIXED (so every 32 rows of it are
+// the same row, and the first one stands for them), and for each of its keys the bias is +0 in every row or -inf in every
+// row.  It then runs the loop of the kernel without bias, with its hidden keys treated like keys that do not exist (their
+// probabilities are 0); every other key block runs in the ordinary biased kernel.
+//
+// The last workgroup writes whether the batch element is a dense one: more than half of a fixed sample of the map (64 of
+// its words, evenly spaced; all of them when the map has at most 64) is MIXED.
+template <typename TB>
+__global__ __launch_bounds__(256) void attn_bias_summary_kernel(const TB* __restrict__ bias, int64_t sb, int64_t sn, int Tq, int Tk,
+                                                                BiasClasses c, uint32_t* __restrict__ info) {
+    typedef typename std::conditional<sizeof(TB) == 2, uint16_t, uint32_t>::type Bits;
+    constexpr Bits NEG = (Bits)(NegInfBits<TB>::value & (sizeof(TB) == 2 ? 0xFFFFu : 0xFFFFFFFFu));
+    __shared__ uint32_t s_and[256], s_or[256], s_any[2], s_open[2];
+    __shared__ int s_ok;
+    const int tid = threadIdx.x, lane = tid & 63, b = blockIdx.y;
+    const int nkb = (Tk + CLS_KEY_BLOCK - 1) / CLS_KEY_BLOCK;
+    uint32_t* out = info + b * c.info_sb;
+    if ((int)blockIdx.x == nkb) {
+        if (tid >= 64) return;
+        const int ntiles = (Tk + CLS_KEYS - 1) / CLS_KEYS;
+        const int total = c.nrow32 * c.nwords;
+        const int i = (int)((int64_t)lane * total / 64);
+        const int w = i % c.nwords;
+        const int n = min(32, ntiles - 32 * w);  // tiles of that word that exist
+        int mixed = cls_count_mixed(c.words[b * c.sb + i], n), seen = n;
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        mixed += __shfl_xor(mixed, off, 64);
-        seen += __shfl_xor(seen, off, 64);
+        for (int off = 32; off > 0; off >>= 1) {
+            mixed += __shfl_xor(mixed, off, 64);
+            seen += __shfl_xor(seen, off, 64);
+        }
+        if (lane == 0) out[0] = 2 * mixed > seen ? 1u : 0u;
+        return;
     }
-    return 2 * mixed > seen;
+    const int kb = blockIdx.x;
+    const int rows32 = min((Tq + CLS_ROWS - 1) / CLS_ROWS, c.nrow32);  // rows of the map that hold query rows
+    const int tile0 = kb * (CLS_KEY_BLOCK / CLS_KEYS);
+    if (tid == 0) s_ok = 1;
+    // no MIXED tile in the two columns of the map: every thread looks at some of the rows
+    bool ok = true;
+    for (int r = tid; r < rows32; r += 256) {
+        const uint32_t v = (uint32_t)(c.words[b * c.sb + (int64_t)r * c.nwords + (tile0 >> 5)] >> (2 * (tile0 & 31)));
+        ok = ok && (v & 3u) != CLS_MIXED && ((v >> 2) & 3u) != CLS_MIXED;
+    }
+    // the first row of every 32, for this thread's key: the two halves of the workgroup take every other one
+    const int key_local = tid & (CLS_KEY_BLOCK - 1), half = tid >> 7;
+    const TB* key_col = bias + b * sb + min(kb * CLS_KEY_BLOCK + key_local, Tk - 1);
+    Bits all_and = (Bits)~(Bits)0, all_or = 0;
+    for (int r0 = half; r0 < rows32; r0 += 32) {
+        Bits v[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+            v[i] = __builtin_bit_cast(Bits, key_col[(int64_t)min(min(r0 + 2 * i, rows32 - 1) * CLS_ROWS, Tq - 1) * sn]);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            all_and &= v[i];
+            all_or |= v[i];
+        }
+    }
+    s_and[tid] = all_and;
+    s_or[tid] = all_or;
+    __syncthreads();
+    if (!ok) atomicAnd(&s_ok, 0);
+    bool hidden = false, good = true;
+    if (tid < CLS_KEY_BLOCK) {
+        const uint32_t a = s_and[tid] & s_and[tid + CLS_KEY_BLOCK], o = s_or[tid] | s_or[tid + CLS_KEY_BLOCK];
+        hidden = a == NEG && o == NEG;
+        good = hidden || o == 0;
+    }
+    const uint64_t hid = __builtin_amdgcn_ballot_w64(hidden);
+    if (__builtin_amdgcn_ballot_w64(!good) != 0 && lane == 0) atomicAnd(&s_ok, 0);
+    uint32_t* e = out + CLS_INFO_HEAD + kb * CLS_INFO_ENTRY;
+    if (tid < CLS_KEY_BLOCK && lane == 0) {
+        e[(tid >> 6) * 2] = (uint32_t)hid;
+        e[(tid >> 6) * 2 + 1] = (uint32_t)(hid >> 32);
+        s_any[tid >> 6] = hid != 0 ? 1u : 0u;        // some key of this half hidden
+        s_open[tid >> 6] = hid != ~0ull ? 1u : 0u;   // some key of this half not hidden
+    }
+    __syncthreads();
+    if (tid == 0) {
+        const bool any_hidden = (s_any[0] | s_any[1]) != 0, any_open = (s_open[0] | s_open[1]) != 0;
+        e[4] = (s_ok != 0 ? CLS_KB_PURE : 0u) | (any_hidden ? CLS_KB_ANY_HIDDEN : 0u) | (!any_open ? CLS_KB_ALL_HIDDEN : 0u);
+    }
 }
 
 // One wavefront classifies a strip of 32 query rows x 8 key tiles (512 keys): every load instruction reads whole rows

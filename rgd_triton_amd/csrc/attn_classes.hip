@@ -9,7 +9,14 @@ static hipError_t classify_launch(const void* bias, int64_t sb, int64_t sn, int 
     const TB* bp = static_cast<const TB*>(bias);
     uint16_t* out = reinterpret_cast<uint16_t*>(words);
     void* args[] = {&bp, &sb, &sn, &Tq, &Tk, const_cast<int*>(&nrow32), const_cast<int*>(&nstrips), &out};
-    return hipLaunchKernel(reinterpret_cast<const void*>(kern), dim3(gx, (unsigned)nb), dim3(256), args, 0, s);
+    hipError_t e = hipLaunchKernel(reinterpret_cast<const void*>(kern), dim3(gx, (unsigned)nb), dim3(256), args, 0, s);
+    if (e != hipSuccess) return e;
+    // the summaries behind the map, from the map and the bias
+    BiasClasses c = cls_layout(words, nb, Tq, Tk);
+    uint32_t* info = const_cast<uint32_t*>(c.info);
+    void (*sum)(const TB*, int64_t, int64_t, int, int, BiasClasses, uint32_t*) = attn_bias_summary_kernel<TB>;
+    void* sargs[] = {&bp, &sb, &sn, &Tq, &Tk, &c, &info};
+    return hipLaunchKernel(reinterpret_cast<const void*>(sum), dim3((unsigned)cls_nkb(Tk) + 1, (unsigned)nb), dim3(256), sargs, 0, s);
 }
 
 // bias: (nb, Tq, Tk) by batch and row strides (elements), 16-byte aligned rows; words: cls_bytes(nb, Tq, Tk) bytes

@@ -134,7 +134,7 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
     if constexpr (HAS_BIAS && DPAD <= 64) {
         // classes came with two launches over the same grid: this one serves the batch elements of its kind
         if (p.cls_take != 0) {
-            if (cls_batch_dense(p.cls, b, (p.Tk + ATTN_BN - 1) / ATTN_BN, lane) != (p.cls_take == 2)) return;
+            if (cls_batch_dense(p.cls, b) != (p.cls_take == 2)) return;
         }
     }
 
