@@ -353,8 +353,8 @@ def attention_case(torch, name, B, T, H, D, dtype, bias_kind, iters=20, with_cpu
     cls_buf = torch.empty(max(cls_bytes, 8) // 8, dtype=torch.int64, device="cuda")
     cls_ptr = cls_buf.data_ptr() if cls_bytes else None
 
-    def fwd():
-        if cls_bytes:
+    def fwd(classify=True):
+        if cls_bytes and classify:
             assert lib.rgd_attn_bias_classify(B, H, T, T, D, bdesc, bk, bd, cls_ptr, cls_bytes, st) == 0, lib.rgd_last_error()
         assert lib.rgd_attn_fwd(B, H, T, T, D, t["q"], t["k"], t["v"], bdesc, bk, bd, t["o"], lse.data_ptr(), code, int(causal),
                                 scale, cls_ptr, fws.data_ptr(), fws.numel(), st) == 0, lib.rgd_last_error()
@@ -382,6 +382,20 @@ def attention_case(torch, name, B, T, H, D, dtype, bias_kind, iters=20, with_cpu
     torch.cuda.synchronize()
     f_ms = statistics.mean(e[0].elapsed_time(e[1]) for e in evs)
     b_ms = statistics.mean(e[1].elapsed_time(e[2]) for e in evs)
+    # the forward when the classes of the bias are already there (a model whose layers share one mask classifies it once
+    # for all of them): reported beside fwd_ms, which includes the classification
+    f_shared = None
+    if cls_bytes:
+        pairs = []
+        for _ in range(iters):
+            a, b_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            fwd(classify=False)
+            b_.record()
+            bwd()
+            pairs.append((a, b_))
+        torch.cuda.synchronize()
+        f_shared = round(statistics.mean(event_ms(pairs)), 4)
     # causal: the pairs above the diagonal do not exist, so half of the dense count is credited
     flops = 14.0 * B * H * T * T * D * (0.5 if causal else 1.0)
     tot = f_ms + b_ms
@@ -395,7 +409,7 @@ def attention_case(torch, name, B, T, H, D, dtype, bias_kind, iters=20, with_cpu
             "frac": round((b_tf if slow_bwd else f_tf) / MFMA_PEAK_TFLOPS, 4),
             "avg_launch_ms": round(b_ms if slow_bwd else f_ms, 4),
             "duration_source": "HIP events around the call, mean of %d" % iters}
-    return {"workload": name, "roofline": roof, "cpu_baseline": cpu, "torch_sdpa": sdpa, "bias_bytes": None if bias is None else bias.numel() * bias.element_size(), "fwd_ms": round(f_ms, 4), "bwd_ms": round(b_ms, 4),
+    return {"workload": name, "roofline": roof, "cpu_baseline": cpu, "torch_sdpa": sdpa, "bias_bytes": None if bias is None else bias.numel() * bias.element_size(), "fwd_ms": round(f_ms, 4), "bwd_ms": round(b_ms, 4), "fwd_ms_classes_given": f_shared,
             "tflops": round(flops / tot / 1e9, 2), "fwd_tflops": round(flops * 4 / 14 / f_ms / 1e9, 2),
             "bwd_tflops": round(flops * 10 / 14 / b_ms / 1e9, 2), "frac_mfma_peak": round(flops / tot / 1e9 / MFMA_PEAK_TFLOPS, 4)}
 

@@ -355,12 +355,17 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
         const int buf = j & 1;
         const int key0 = j * BN;
         const bool tail = !F && key0 + BN > L.Tk;
-        if (F || j + 1 < run_end) {
-            if constexpr (AH == 0) issue_loads(j + 1, FAST, IntC<0>{});
-            else issue_loads(j + 2, FAST, IntC<AH - 1>{});
-            if constexpr (BIAS_AHEAD)
-                bias_nxt.load(bias_row, key0 + BN, g, L.Tk, F || (p.bias_vec && key0 + 2 * BN <= L.Tk));
-        }
+        // the fetch of the next tile(s).  CLS: issued inside either arm of the class test below, so that each arm is one
+        // block of loads, address arithmetic, products and the first use of their results, as in the kernel without bias
+        auto fetch = [&]() __attribute__((always_inline)) {
+            if (F || j + 1 < run_end) {
+                if constexpr (AH == 0) issue_loads(j + 1, FAST, IntC<0>{});
+                else issue_loads(j + 2, FAST, IntC<AH - 1>{});
+                if constexpr (BIAS_AHEAD)
+                    bias_nxt.load(bias_row, key0 + BN, g, L.Tk, F || (p.bias_vec && key0 + 2 * BN <= L.Tk));
+            }
+        };
+        if constexpr (!CLS) fetch();
         // WB: the tile has a bias: the registers fetched a step ago, or (CLS: a run of MIXED tiles, which are few) read
         // here, at the start of the tile's own step
         auto body = [&](auto WB) __attribute__((always_inline)) {
@@ -405,6 +410,13 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
                 }
             }
         };
+        // t = logit - lse (log2 domain), for tiles whose bias, if any, is already inside s
+        auto logits = [&]() __attribute__((always_inline)) {
+#pragma unroll
+            for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) s[kb][v] = fmaf(s[kb][v], L.scale_log2, neg_lse_l2);
+        };
         auto from_zero = [&]() __attribute__((always_inline)) {
 #pragma unroll
             for (int kb = 0; kb < NKB; ++kb)
@@ -419,13 +431,22 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
             // for the same reason.  COLUMN: every row of the tile is the first row of this wavefront's 32, which all its
             // lanes read.  The products are written out twice, so that the one that starts from zero keeps its zero inside
             // its first matrix instructions instead of in 32 registers that something has to clear.
-            if (__builtin_expect(tc != CLS_ZERO, 0)) {
-                int row = tc == CLS_COLUMN ? min(qb * BWD_BM + wave * 32, L.Tq - 1) : q_ld;
+            if (__builtin_expect(tc == CLS_ZERO, 1)) {
+                fetch();
+                from_zero();
+                logits();
+            } else {
+                // (the class as a value of its own: the compiler otherwise threads the choice of the row through the test
+                // above, which puts four branches in front of every tile)
+                int tcc = tc;
+                asm volatile("" : "+s"(tcc));
+                int row = tcc == CLS_COLUMN ? min(qb * BWD_BM + wave * 32, L.Tq - 1) : q_ld;
                 asm volatile("" : "+v"(row));
                 // the bias tensor is read from the kernel's argument memory here, not kept in scalar registers through the loop
                 const AttnTensor& bt = cold_params<AttnBwdParams>().bias;
                 const TB* here = static_cast<const TB*>(bt.ptr) + b * bt.sb + h * bt.sh + (int64_t)row * bt.sn;
                 const float per_score = kLog2e / L.scale_log2;
+                fetch();
 #pragma unroll
                 for (int kb = 0; kb < NKB; ++kb) {
                     BiasRuns<TB, 1> half;
@@ -436,9 +457,8 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
                     for (int v = 0; v < 16; ++v) s[kb][v] = bias_h[v] * per_score;
                 }
                 products();
+                logits();
                 asm volatile("" ::: "memory");  // (keeps the two copies apart)
-            } else {
-                from_zero();
             }
         } else {
             from_zero();
@@ -455,7 +475,7 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
         }
         if (!masked_tile) {
         // t = logit - lse (log2 domain)
-        {
+        if constexpr (!CLS) {
             float bias_v[NKB][16];
             if constexpr (WITH_BIAS && !CLS) bias_use.decode(bias_v);
 #pragma unroll

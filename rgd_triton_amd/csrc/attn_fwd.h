@@ -292,12 +292,17 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
         const int buf = j & 1;
         const int key0 = j * ATTN_BN;
         const bool tail = !F && key0 + ATTN_BN > L.Tk;
-        if (F || j + 1 < run_end) {
-            if constexpr (AH == 0) issue_loads(j + 1, FAST, IntC<0>{});
-            else issue_loads(j + 2, FAST, IntC<AH - 1>{});
-            if constexpr (BIAS_AHEAD)
-                bias_nxt.load(bias_row, key0 + ATTN_BN, g, L.Tk, F || (p.bias_vec && key0 + 2 * ATTN_BN <= L.Tk));
-        }
+        // the fetch of the next tile(s).  CLS, d <= 64: issued inside either arm of the class test below, so that each arm
+        // is one block of loads, address arithmetic, product and the first use of its result, as in the kernel without bias
+        auto fetch = [&]() __attribute__((always_inline)) {
+            if (F || j + 1 < run_end) {
+                if constexpr (AH == 0) issue_loads(j + 1, FAST, IntC<0>{});
+                else issue_loads(j + 2, FAST, IntC<AH - 1>{});
+                if constexpr (BIAS_AHEAD)
+                    bias_nxt.load(bias_row, key0 + ATTN_BN, g, L.Tk, F || (p.bias_vec && key0 + 2 * ATTN_BN <= L.Tk));
+            }
+        };
+        if constexpr (!(CLS && !SPLIT_HALVES)) fetch();
         if constexpr (!SPLIT_HALVES) {
             // d <= 64: both 32-key halves of the tile go through the softmax together.
             // WB: the tile has a bias: the registers fetched a step ago, or (CLS, a MIXED tile) read here.
@@ -325,6 +330,14 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
                     for (int v = 0; v < 16; ++v) s[kb][v] = 0.f;
                 products();
             };
+            // t = logit - m_ref (log2 domain), for tiles whose bias, if any, is already inside s
+            const float m_off = m_ref == -INFINITY ? 0.f : m_ref;
+            auto logits = [&]() __attribute__((always_inline)) {
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) s[kb][v] = fmaf(s[kb][v], L.scale_log2, -m_off);
+            };
             if constexpr (CLS) {
                 // A MIXED or COLUMN tile (few; tc is its class): the product starts from the bias, in units of the raw
                 // scores, instead of from zero, and the tile goes on like every other tile.  The bias is read here, straight
@@ -334,13 +347,22 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
                 // zero inside its first matrix instructions instead of in 32 registers that something has to clear.
                 // (A copy of the whole step for these tiles, which would leave the step of the other tiles exactly that of
                 // the kernel without bias, costs that step registers it does not have: spills.)
-                if (__builtin_expect(tc != CLS_ZERO, 0)) {
-                    int row = tc == CLS_COLUMN ? min(qb * ATTN_BM + wave * 32, L.Tq - 1) : q_ld;
+                if (__builtin_expect(tc == CLS_ZERO, 1)) {
+                    fetch();
+                    from_zero();
+                    logits();
+                } else {
+                    // (the class as a value of its own: the compiler otherwise threads the choice of the row through the
+                    // test above, which puts four branches in front of every tile)
+                    int tcc = tc;
+                    asm volatile("" : "+s"(tcc));
+                    int row = tcc == CLS_COLUMN ? min(qb * ATTN_BM + wave * 32, L.Tq - 1) : q_ld;
                     asm volatile("" : "+v"(row));
                     // the bias tensor is read from the kernel's argument memory here, not kept in scalar registers through the loop
                     const AttnTensor& bt = cold_params<AttnFwdParams>().bias;
                     const TB* here = static_cast<const TB*>(bt.ptr) + b * bt.sb + h * bt.sh + (int64_t)row * bt.sn;
                     const float per_score = kLog2e / L.scale_log2;
+                    fetch();
 #pragma unroll
                     for (int kb = 0; kb < 2; ++kb) {
                         BiasRuns<TB, 1> half;
@@ -351,19 +373,19 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
                         for (int v = 0; v < 16; ++v) s[kb][v] = bias_v[v] * per_score;
                     }
                     products();
+                    logits();
                     asm volatile("" ::: "memory");  // (keeps the two copies apart)
-                } else {
-                    from_zero();
                 }
             } else {
                 from_zero();
             }
 
             // ---- t = logit - m_ref (log2 domain) ----
-            const float m_off = m_ref == -INFINITY ? 0.f : m_ref;
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb) {
-                if constexpr (WITH_BIAS && !CLS) {
+                if constexpr (CLS) {
+                    // (done in either arm above)
+                } else if constexpr (WITH_BIAS) {
                     float bias_v[16];
                     bias_use.decode_run(kb, bias_v);
 #pragma unroll

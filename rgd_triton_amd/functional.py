@@ -490,6 +490,21 @@ def _bias_args(bias, q, seqlen_q, seqlen_k, batch, nheads):
     return desc, kind, _hip.dtype_code(bias.dtype)
 
 
+# The classes of the last head-shared bias seen on each device.  The layers of a model usually share one mask: the first
+# attention call of a step classifies it, the others find the classes here.  An entry names the bias by its storage,
+# view and version counter (in-place writes through any view bump it) and holds the storage, so that its address cannot
+# be given to another tensor while the entry lives; one entry per device, replaced by the next bias.
+# Writes that bypass the counter (through `.data`, or by a kernel that was handed the raw pointer) are not seen: call
+# clear_bias_classes_cache() after them, or set RGD_CLASSES_CACHE=0.
+_classes_cache = {}
+_classes_cache_on = os.environ.get("RGD_CLASSES_CACHE", "1") != "0"
+
+
+def clear_bias_classes_cache():
+    """Forgets the tile classes kept for the last head-shared attention bias of every device."""
+    _classes_cache.clear()
+
+
 def _bias_classes(bias, bdesc, bkind, bdtype, dims):
     """Tile classes of a bias matrix that the heads share (rgd_attn_bias_classify): one pass over the bias, made in the
     forward and kept for the backward.  None when the library has no use for them (any other bias, head dims above 64)."""
@@ -499,9 +514,21 @@ def _bias_classes(bias, bdesc, bkind, bdtype, dims):
     nbytes = lib.rgd_attn_bias_classes_bytes(*dims, bdesc, bkind, bdtype)
     if nbytes == 0:
         return None
+    # under stream capture the classification must be part of the graph (a replay may find new values in the bias)
+    cacheable = _classes_cache_on and not torch.cuda.is_current_stream_capturing()
+    storage = bias.untyped_storage()
+    # (the stream too: the classes are ready for work queued behind them on the stream that wrote them)
+    key = (storage.data_ptr(), bias.storage_offset(), tuple(bias.shape), tuple(bias.stride()), bias.dtype, bias._version, dims,
+           torch.cuda.current_stream(bias.device).cuda_stream)
+    if cacheable:
+        hit = _classes_cache.get(bias.device)
+        if hit is not None and hit[0] == key:
+            return hit[2]
     classes = torch.empty(nbytes // 8, dtype=torch.int64, device=bias.device)
     _hip.check(lib.rgd_attn_bias_classify(*dims, bdesc, bkind, bdtype, classes.data_ptr(), nbytes, _hip.stream_ptr(bias.device)),
                "rgd_attn_bias_classify")
+    if cacheable:
+        _classes_cache[bias.device] = (key, storage, classes)
     return classes
 
 

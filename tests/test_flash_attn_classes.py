@@ -1,5 +1,7 @@
 """Tile classes of a head-shared attention bias (rgd_attn_bias_classify and the kernels that read the classes): results
-must equal the ordinary biased kernels bit for bit, and the oracle within the reference's tolerance."""
+must equal those of the ordinary biased kernels (bit for bit for a dense bias, which those kernels still serve, and for an
+all-zero one against a call without bias; to the last bits of the tensor type otherwise, because the bias enters the
+logits before the product instead of after it), and the oracle within the reference's tolerance."""
 import math
 
 import pytest
@@ -165,3 +167,47 @@ def test_flash_attn_zero_bias_equals_no_bias(d, dtype):
     for a, b, n in zip(outs[0], outs[1], ("o", "lse", "dq", "dk", "dv")):
         it = torch.int16 if a.element_size() == 2 else torch.int32
         assert torch.equal(a.view(it), b.view(it)), n
+
+
+def test_flash_attn_shared_mask_classes_are_reused_and_follow_the_mask():
+    """Through the Module API: the layers of a model that share one mask classify it once (the second call finds the
+    classes of the first), an in-place change of the mask is seen (version counter), and forward + backward through
+    autograd agree with the oracle either way."""
+    from rgd_triton_amd import FlashAttention, clear_bias_classes_cache, functional
+
+    g = gen(21)
+    B, H, T, d, dtype = 2, 4, 320, 64, torch.bfloat16
+    q, k, v, do = (randn(g, B, T, H, d, dtype=dtype) for _ in range(4))
+    mask = torch.zeros(B, 1, T, T)
+    mask[0, :, :, 250:] = float("-inf")
+    mask[1, :, :, 300:] = float("-inf")
+    mask = mask.to(dtype)
+    attn = FlashAttention()
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    mg = mask.cuda()
+
+    def run():
+        o = attn(qg, kg, vg, bias=mg)
+        return (o, *torch.autograd.grad(o, (qg, kg, vg), do.cuda()))
+
+    def check(got, m):
+        o_ref, _ = oracle.attention_fwd(q, k, v, m)
+        g_ref = oracle.attention_bwd(do, q, k, v, m, False, None)
+        for a, b in zip(got, (o_ref, *g_ref[:3])):
+            assert (a.float().cpu() - b.float()).abs().max().item() < 3e-2
+
+    clear_bias_classes_cache()
+    first = run()
+    entry = functional._classes_cache[mg.device]
+    second = run()
+    assert functional._classes_cache[mg.device][2] is entry[2]  # found, not written again
+    for a, b in zip(first, second):
+        assert torch.equal(a, b)
+    check(first, mask)
+    # the mask changes in place: other keys are hidden now
+    mg[:, :, :, 100:164] = float("-inf")
+    mask2 = mg.cpu()
+    third = run()
+    assert functional._classes_cache[mg.device][2] is not entry[2]
+    check(third, mask2)
+    assert not torch.equal(third[0], first[0])
