@@ -222,8 +222,8 @@ int rgd_ln_rope_qk_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D,
  * them (flash_attn/flash_attn_triton_cached.py:790-792) */
 int64_t rgd_attn_seqlen_q_rounded(int64_t Tq);
 
-/* Tile classes of a bias matrix that the heads share (stride_h == 0), head dims up to 64.  Such a bias is usually a
- * mask (0 / -inf), and the reference streams it tile by tile for every head and in every kernel
+/* Tile classes of a bias, matrix or vector, that the heads share (stride_h == 0), head dims up to 64.  Such a bias is
+ * usually a mask (0 / -inf), and the reference streams it tile by tile for every head and in every kernel
  * (flash_attn/flash_attn_triton_cached.py:151-175, :430-470).  One pass over the matrix leaves two bits per tile of 32
  * queries x 64 keys (all +0; all -inf; every row equal to the tile's first row; anything else); rgd_attn_fwd and
  * rgd_attn_bwd then run tiles that are all +0 like tiles without bias, leave all -inf tiles out and read the bias only
@@ -231,13 +231,13 @@ int64_t rgd_attn_seqlen_q_rounded(int64_t Tq);
  * bit for bit.  In tiles that read the bias, the bias enters the logits before the q.k product is added instead of
  * after it, and the dQ kernel adds do.v^T to -delta instead of subtracting delta afterwards: against a call that uses no
  * classes, o, lse, dq, dk and dv agree to the last one or two bits of the tensor dtype, not bit for bit (a call is
- * still reproducible bit for bit against itself).  Batch elements whose tiles are mostly of the last kind are run by
- * the ordinary kernels, bit for bit as without classes.  Both calls make the pass themselves, into the end of their
+ * still reproducible bit for bit against itself).  Batch elements in most of whose tiles the bias has to be read are run
+ * by the ordinary kernels, bit for bit as without classes.  Both calls make the pass themselves, into the end of their
  * workspace, when bias_classes is NULL; a caller that runs several calls on one bias (a forward and its backward, or
  * every layer of a model that shares one mask) can make it once:
  *   rgd_attn_bias_classes_bytes  size of the classes for this bias and shape; 0 when they would not be used
- *                                (bias not a matrix, not shared by the heads, rows not 16-byte aligned, D > 64, H < 2)
- *   rgd_attn_bias_classify       writes them (8-byte aligned buffer of that size), one kernel launch on `stream`
+ *                                (no bias, not shared by the heads, rows not 16-byte aligned, D > 64, H < 2, Tk < 64)
+ *   rgd_attn_bias_classify       writes them (8-byte aligned buffer of that size), two kernel launches on `stream`
  * and pass the buffer as bias_classes.  The classes describe the bias VALUES: classify again when they change. */
 size_t rgd_attn_bias_classes_bytes(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D,
                                    const rgd_tensor4* bias, int bias_kind, int bias_dtype);

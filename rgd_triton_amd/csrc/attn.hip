@@ -69,13 +69,17 @@ bool bwd_one_pass(int mode, int64_t D, size_t workspace_bytes, size_t need) {
     return RGD_ATTN_BWD_AUTO_ONE_PASS && workspace_bytes >= need;
 }
 
-// Tile classes (attn_classes.h) pay for a bias matrix that several heads share: one pass over it instead of one per
-// head and kernel.  Head dims up to 64 (the kernels for wider heads have no registers for a second code path), rows the
-// 16-byte loads can read, and a key count a wavefront can keep the classes of.
+// a vector bias is a matrix whose rows are all the same row
+int64_t cls_row_stride(const rgd_tensor4* bias, int bias_kind) { return bias_kind == RGD_BIAS_VECTOR ? 0 : bias->stride_n; }
+// Tile classes (attn_classes.h) pay for a bias (matrix or vector) that several heads share: one pass over it instead of
+// one per head and kernel.  Head dims up to 64 (the kernels for wider heads have no registers for a second code path),
+// rows the 16-byte loads can read, and a key count a wavefront can keep the classes of.
 bool cls_eligible(int64_t H, int64_t Tq, int64_t Tk, int64_t D, const rgd_tensor4* bias, int bias_kind, int bias_dtype) {
-    if (bias_kind != RGD_BIAS_MATRIX || !bias || bias->stride_h != 0 || H < 2 || D > 64 || Tq < 1 || Tk < CLS_KEYS) return false;
+    if ((bias_kind != RGD_BIAS_MATRIX && bias_kind != RGD_BIAS_VECTOR) || !bias || bias->stride_h != 0 || H < 2 || D > 64 || Tq < 1 ||
+        Tk < CLS_KEYS)
+        return false;
     const int64_t per16 = bias_dtype == RGD_F32 ? 4 : 8;
-    if (!rgd_aligned16(bias->ptr) || bias->stride_b % per16 != 0 || bias->stride_n % per16 != 0) return false;
+    if (!rgd_aligned16(bias->ptr) || bias->stride_b % per16 != 0 || cls_row_stride(bias, bias_kind) % per16 != 0) return false;
     return cls_nwords(Tk) <= CLS_MAX_WORDS && cls_nrow32(Tq) <= CLS_MAX_ROWS;
 }
 int64_t cls_batches(int64_t B, const rgd_tensor4* bias) { return bias->stride_b == 0 ? 1 : B; }
@@ -102,7 +106,7 @@ const void* cls_for_call(const char* name, int64_t B, int64_t H, int64_t Tq, int
     const size_t tail = (workspace_bytes - need) & ~(size_t)15;
     if (reinterpret_cast<uintptr_t>(workspace) & 7u) return nullptr;
     uint64_t* words = reinterpret_cast<uint64_t*>(static_cast<char*>(workspace) + tail);
-    *rc = attn_classify(bias->ptr, bias->stride_b, bias->stride_n, bias_dtype, (int)cls_batches(B, bias), Tq, Tk, words, s);
+    *rc = attn_classify(bias->ptr, bias->stride_b, cls_row_stride(bias, bias_kind), bias_dtype, (int)cls_batches(B, bias), Tq, Tk, words, s);
     if (*rc != RGD_OK) return nullptr;
     *room = tail;
     return words;
@@ -164,7 +168,7 @@ int rgd_attn_bias_classify(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t
     RGD_REQUIRE(need > 0, RGD_ERR_UNSUPPORTED, "%s: no tile classes for this bias and shape (rgd_attn_bias_classes_bytes is 0)", name);
     RGD_REQUIRE(classes && (reinterpret_cast<uintptr_t>(classes) & 7u) == 0 && classes_bytes >= need, RGD_ERR_WORKSPACE,
                 "%s: classes needs %zu bytes, 8-byte aligned", name, need);
-    return attn_classify(bias->ptr, bias->stride_b, bias->stride_n, bias_dtype, (int)cls_batches(B, bias), Tq, Tk,
+    return attn_classify(bias->ptr, bias->stride_b, cls_row_stride(bias, bias_kind), bias_dtype, (int)cls_batches(B, bias), Tq, Tk,
                          static_cast<uint64_t*>(classes), static_cast<hipStream_t>(stream));
 }
 

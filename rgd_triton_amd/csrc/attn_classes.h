@@ -31,7 +31,7 @@ constexpr int CLS_INFO_ENTRY = 8;      // 32-bit words per key block entry
 
 // Behind the map lies a summary per batch element, written by a second launch (attn_bias_summary_kernel), so that no
 // workgroup of the attention kernels has to derive it again:
-//     info[b * info_sb + 0]                             1: most tiles are MIXED, the ordinary biased kernels serve b
+//     info[b * info_sb + 0]                             1: most tiles have to be read, the ordinary biased kernels serve b
 //     info[b * info_sb + CLS_INFO_HEAD + kb * 8 + 0..3]  key block kb (128 keys): bit k set = key k is hidden from every query
 //     info[b * info_sb + CLS_INFO_HEAD + kb * 8 + 4]     bit 0: "key mask" block (see attn_bias_summary_kernel), bit 1: some key
 //                                                       of it is hidden, bit 2: every key of it is
@@ -90,11 +90,11 @@ __device__ __forceinline__ void cls_tiles_to_lds(const BiasClasses& c, int b, in
 // class of tile / step j, the same value in every lane (a scalar for the compiler)
 __device__ __forceinline__ int cls_lds_at(const uint8_t* lds, int j) { return __builtin_amdgcn_readfirstlane((int)lds[j]); }
 
-// number of MIXED tiles among the first n tiles of a word
-__device__ __forceinline__ int cls_count_mixed(uint64_t w, int n) {
-    const uint64_t any = (w | (w >> 1)) & 0x5555555555555555ull;  // bit 2t set: tile t is not MIXED
+// number of tiles among the first n of a word whose bias has to be read (MIXED or COLUMN: both bits alike)
+__device__ __forceinline__ int cls_count_read(uint64_t w, int n) {
+    const uint64_t alike = ~(w ^ (w >> 1)) & 0x5555555555555555ull;  // bit 2t set: tile t is MIXED (00) or COLUMN (11)
     const uint64_t keep = n >= 32 ? ~0ull : ((1ull << (2 * n)) - 1);
-    return n - (int)__builtin_popcountll(any & keep);
+    return (int)__builtin_popcountll(alike & keep);
 }
 
 // Which kernels serve a batch element.  A bias with classes is launched twice over the same grid: the CLS variant of
@@ -118,8 +118,8 @@ __device__ __forceinline__ const uint32_t* cls_key_block(const BiasClasses& c, i
 // row.  It then runs the loop of the kernel without bias, with its hidden keys treated like keys that do not exist (their
 // probabilities are 0); every other key block runs in the ordinary biased kernel.
 //
-// The last workgroup writes whether the batch element is a dense one: more than half of a fixed sample of the map (64 of
-// its words, evenly spaced; all of them when the map has at most 64) is MIXED.
+// The last workgroup writes whether the batch element is a dense one: in more than half of a fixed sample of the map (64
+// of its words, evenly spaced; all of them when the map has at most 64) the bias has to be read (MIXED or COLUMN tiles).
 template <typename TB>
 __global__ __launch_bounds__(256) void attn_bias_summary_kernel(const TB* __restrict__ bias, int64_t sb, int64_t sn, int Tq, int Tk,
                                                                 BiasClasses c, uint32_t* __restrict__ info) {
@@ -137,7 +137,7 @@ __global__ __launch_bounds__(256) void attn_bias_summary_kernel(const TB* __rest
         const int i = (int)((int64_t)lane * total / 64);
         const int w = i % c.nwords;
         const int n = min(32, ntiles - 32 * w);  // tiles of that word that exist
-        int mixed = cls_count_mixed(c.words[b * c.sb + i], n), seen = n;
+        int mixed = cls_count_read(c.words[b * c.sb + i], n), seen = n;
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) {
             mixed += __shfl_xor(mixed, off, 64);

@@ -42,6 +42,10 @@ def _mask(kind, B, Tq, Tk, g, dtype):
         m[:, :, :, 0] = 0
     elif kind == "dense":
         m = 0.5 * torch.randn(B, 1, Tq, Tk, generator=g)
+    elif kind == "vpadding":  # the padding mask as a (B, 1, 1, Tk) vector
+        return _mask("padding", B, Tq, Tk, g, dtype)[:, :, :1].contiguous()
+    elif kind == "vdense":  # a finite value per key
+        return 0.5 * torch.randn(B, 1, 1, Tk, generator=g)
     elif kind == "negzero":  # -0.0 is not +0.0 for the classes: such tiles must take the general path
         m = -m
     elif kind == "hidden_rows":  # some query rows see no key at all
@@ -65,6 +69,9 @@ CASES = [
     ("negzero", 1, 2, 128, 128, 64, None, False, False),
     ("hidden_rows", 1, 2, 256, 192, 64, None, False, False),
     ("padding", 2, 4, 4352 // 4, 4352 // 4, 64, None, False, False),
+    ("vpadding", 2, 4, 512, 640, 64, None, False, False),
+    ("vpadding", 2, 3, 300, 777, 32, torch.float32, False, False),
+    ("vdense", 2, 4, 256, 320, 64, None, False, False),
 ]
 
 
@@ -81,11 +88,12 @@ def test_flash_attn_bias_classes(case, dtype):
     qg, kg, vg, dog = (x.cuda() for x in (q, k, v, do))
     # rows the 16-byte loads can read: a view into a buffer whose rows are padded to 16 elements
     tk_pad = (Tk + 15) // 16 * 16
-    bg = torch.full((bias.shape[0], 1, Tq, tk_pad), float("nan"), dtype=bias.dtype, device="cuda")[..., :Tk]
+    bg = torch.full((bias.shape[0], 1, bias.shape[2], tk_pad), float("nan"), dtype=bias.dtype, device="cuda")[..., :Tk]
     bg.copy_(bias)
     be = bg.expand(B, H, Tq, Tk)
     bdesc = _hip.Tensor4(be.data_ptr(), be.stride(0), be.stride(1), be.stride(2))
-    bk, bd, code = _hip.BIAS_MATRIX, _hip.dtype_code(bg.dtype), _hip.dtype_code(dtype)
+    bk = _hip.BIAS_VECTOR if bias.shape[2] == 1 else _hip.BIAS_MATRIX
+    bd, code = _hip.dtype_code(bg.dtype), _hip.dtype_code(dtype)
     scale = 1.0 / math.sqrt(d)
     st = _hip.stream_ptr(qg.device)
     tqr = lib.rgd_attn_seqlen_q_rounded(Tq)
@@ -116,12 +124,12 @@ def test_flash_attn_bias_classes(case, dtype):
         return dict(o=o, lse=lse[:, :, :Tq], dq=dq, dk=dk, dv=dv)
 
     plain, given = run(0), run(1)
-    # A bias that is mostly MIXED tiles (the dense one) is handed to the ordinary kernels: the same bits.  Otherwise ZERO
+    # A bias that is mostly MIXED or COLUMN tiles (the dense ones) is handed to the ordinary kernels: the same bits.  Otherwise ZERO
     # tiles run the instructions of a tile without bias (the same bits again), NEG tiles are left out (they add exact
     # zeros), and on a MIXED or COLUMN tile (the -0.0 bias is all COLUMN tiles) the first product starts from the bias in
     # units of the raw scores (one rounding apart from adding it after the scaling), so results agree to rounding, not to
     # the bit.
-    exact = kind == "dense"
+    exact = kind in ("dense", "vdense")
     ulp = 2.0 ** (-7 if dtype == torch.bfloat16 else -10)
     for n in plain:
         a, b = plain[n], given[n]
