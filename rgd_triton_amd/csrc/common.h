@@ -134,6 +134,29 @@ __device__ __forceinline__ void store_chunk(T* __restrict__ p, int first, int li
     }
 }
 
+// 16-byte path: N floats -> `base + byte_off` (uniform base, 32-bit offset per lane), if `ok`
+template <typename T, int N, bool NT = false>
+__device__ __forceinline__ void store_chunk_at(void* __restrict__ base, uint32_t byte_off, bool ok, const float (&in)[N]) {
+    static_assert((N * sizeof(T)) % 16 == 0, "store_chunk_at: 16-byte chunks");
+    constexpr int NV = N * sizeof(T) / 16;
+    constexpr int EPV = 16 / sizeof(T);
+    if (ok) {
+        u32x4* vp = reinterpret_cast<u32x4*>(static_cast<char*>(base) + byte_off);
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            T tmp[EPV];
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) tmp[e] = from_f32<T>(in[v * EPV + e]);
+            u32x4 raw;
+            __builtin_memcpy(&raw, tmp, 16);
+            if constexpr (NT)
+                __builtin_nontemporal_store(raw, vp + v);
+            else
+                vp[v] = raw;
+        }
+    }
+}
+
 // Branch-free variant used in the streaming loops: the load is unconditional (a chunk that is out of
 // range reads the start of the row instead, which is always valid memory) and out-of-range elements are
 // zeroed by a select when the raw bits are decoded.  Issue every load() of an iteration first, then
@@ -161,6 +184,19 @@ template <typename T, int N, bool VECTOR, bool NT = false> struct Chunk {
         } else {
 #pragma unroll
             for (int e = 0; e < N; ++e) s[e] = row[first + e < limit ? first + e : 0];
+        }
+    }
+    // 16-byte path only: the chunk at `base + byte_off`, a uniform base and a 32-bit offset per lane (the address
+    // arithmetic stays in 32 bits and the load takes the base from scalar registers)
+    __device__ __forceinline__ void load_at(const void* __restrict__ base, uint32_t byte_off) {
+        static_assert(VEC, "load_at: 16-byte chunks");
+        const u32x4* p = reinterpret_cast<const u32x4*>(static_cast<const char*>(base) + byte_off);
+#pragma unroll
+        for (int i = 0; i < NVEC; ++i) {
+            if constexpr (NT)
+                v[i] = __builtin_nontemporal_load(p + i);
+            else
+                v[i] = p[i];
         }
     }
     // MASK = false skips the zeroing selects (the caller knows every element is in range)

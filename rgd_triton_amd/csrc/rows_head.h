@@ -27,6 +27,9 @@ struct HeadHalf {
     uint32_t n12, n2;
     int token_is_inner;  // the inner index is the token (else the head)
     int cutoff;          // tokens >= cutoff are not rotated
+    // COMPACT launches: the rows of x, dy and y lie at equal distances in iteration order (row r at r * bytes), and every
+    // byte offset fits 31 bits
+    uint32_t rbx, rbd, rby;
 };
 
 #ifndef RGD_HEAD_PERSIST
@@ -46,12 +49,18 @@ struct HeadParams {
     int64_t pe_ss, pe_sn;
     int R;
     int rope_bwd;  // flip the rotation sign
+    uint32_t pe_row_bytes, pe_cos_bytes;  // COMPACT launches: bytes between table rows, and from the sin to the cos table
 };
 
 // T = tensor element type, TP = rotary table element type (T or float)
 // FULL: D == G*NV*VEC, so no element of a lane's chunks is ever out of range
-template <typename T, typename TP, int MODE, int G, int NV, int VEC, bool VECTOR, bool FULL, int U>
+// COMPACT (with VECTOR and FULL): addresses are a uniform base plus a 32-bit byte offset per lane, row r of a tensor at
+// r * its row distance.  The general form spends a quarter of its vector instructions on 64-bit address arithmetic
+// (three 64-bit multiply-adds per tensor and row), and these kernels are bound by vector instruction issue as much as by
+// memory: at 16 bytes per lane and row there are 160-240 instructions per row.
+template <typename T, typename TP, int MODE, int G, int NV, int VEC, bool VECTOR, bool FULL, int U, bool COMPACT = false>
 __global__ __launch_bounds__(256) void head_rows_kernel(const HeadParams p) {
+    static_assert(!COMPACT || (VECTOR && FULL), "COMPACT: whole 16-byte chunks");
     constexpr bool HAS_LN = MODE != HEAD_ROPE;
     constexpr bool HAS_ROPE = MODE == HEAD_ROPE || MODE == HEAD_LNROPE_FWD || MODE == HEAD_LNROPE_BWD;
     constexpr bool BWD = MODE == HEAD_LN_BWD || MODE == HEAD_LNROPE_BWD;
@@ -77,6 +86,10 @@ __global__ __launch_bounds__(256) void head_rows_kernel(const HeadParams p) {
     bool rotate[U];
     int lim[U];
     T* yrow[U];
+    uint32_t yoff[U];  // COMPACT
+    // COMPACT: this lane's bytes inside a row, and inside a table row (lanes past the rotary channels read its start)
+    const uint32_t lane_bytes = (uint32_t)(lg * VEC) * (uint32_t)sizeof(T);
+    const uint32_t lane_pe_bytes = (uint32_t)(lg * VEC < p.R ? lg * VEC : 0) * (uint32_t)sizeof(TP);
 
     // ---- phase 1: addresses and loads ----
 #pragma unroll
@@ -91,6 +104,31 @@ __global__ __launch_bounds__(256) void head_rows_kernel(const HeadParams p) {
         const int token = h.token_is_inner ? (int)i2 : (int)i1;
         lim[u] = valid ? D : 0;
         rotate[u] = HAS_ROPE && valid && token < h.cutoff;
+        if constexpr (COMPACT) {
+            constexpr uint32_t KSTEP = (uint32_t)(G * VEC) * (uint32_t)sizeof(T);
+            const uint32_t xoff = __umul24(r, h.rbx) + lane_bytes;  // both below 2^24 (checked on the host)
+            yoff[u] = __umul24(r, h.rby) + lane_bytes;
+#pragma unroll
+            for (int k = 0; k < NV; ++k) xc[u][k].load_at(h.x, xoff + k * KSTEP);
+            if constexpr (BWD) {
+                const uint32_t doff = __umul24(r, h.rbd) + lane_bytes;
+#pragma unroll
+                for (int k = 0; k < NV; ++k) dc[u][k].load_at(h.dy, doff + k * KSTEP);
+            }
+            if constexpr (HAS_ROPE) {
+                const uint32_t poff = __umul24((uint32_t)token, p.pe_row_bytes) + lane_pe_bytes;
+                const char* cos_base = static_cast<const char*>(p.pe) + p.pe_cos_bytes;
+#pragma unroll
+                for (int k = 0; k < NV; ++k) {
+                    // chunk k of a lane starts at channel (k*G + lg)*VEC; past the rotary channels it reads the row's start
+                    const uint32_t pk = (k == 0) ? poff
+                                                 : __umul24((uint32_t)token, p.pe_row_bytes) +
+                                                       (uint32_t)((k * G + lg) * VEC < p.R ? (k * G + lg) * VEC : 0) * (uint32_t)sizeof(TP);
+                    sc[u][k].load_at(p.pe, pk);
+                    cc[u][k].load_at(cos_base, pk);
+                }
+            }
+        } else {
         const T* xr = static_cast<const T*>(h.x) + (int64_t)b * h.sx[0] + (int64_t)i1 * h.sx[1] + (int64_t)i2 * h.sx[2];
         yrow[u] = static_cast<T*>(h.y) + (int64_t)b * h.sy[0] + (int64_t)i1 * h.sy[1] + (int64_t)i2 * h.sy[2];
 #pragma unroll
@@ -100,7 +138,8 @@ __global__ __launch_bounds__(256) void head_rows_kernel(const HeadParams p) {
 #pragma unroll
             for (int k = 0; k < NV; ++k) dc[u][k].load(dr, (k * G + lg) * VEC, D);
         }
-        if constexpr (HAS_ROPE) {
+        }
+        if constexpr (HAS_ROPE && !COMPACT) {
             // token < T < P always holds, so the table row exists even for rows that are not rotated
             const TP* sin_row = static_cast<const TP*>(p.pe) + (int64_t)token * p.pe_sn;
             const TP* cos_row = sin_row + p.pe_ss;
@@ -139,10 +178,14 @@ __global__ __launch_bounds__(256) void head_rows_kernel(const HeadParams p) {
                     ss += xcen * xcen;
                 }
             rstd = rsqrtf(group_reduce<G>(ss) * p.inv_d + p.eps);
+            // forward: xhat.  The backward keeps the centred x and folds rstd into its three row constants below
+            // (two instructions per element less).
+            if constexpr (!BWD) {
 #pragma unroll
-            for (int k = 0; k < NV; ++k)
+                for (int k = 0; k < NV; ++k)
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) xv[k][e] *= rstd;  // xhat
+                    for (int e = 0; e < VEC; ++e) xv[k][e] *= rstd;
+            }
         }
         if constexpr (HAS_ROPE) {
             // forward rotation (x0, x1) -> (-x1, x0); the backward uses (x1, -x0).  sin and cos are
@@ -183,15 +226,23 @@ __global__ __launch_bounds__(256) void head_rows_kernel(const HeadParams p) {
                     si += xv[k][e] * dv[k][e];
                     sg += dv[k][e];
                 }
-            const float inner = group_reduce<G>(si) * p.inv_d;
+            // dx = (dy - xhat * mean(xhat dy) - mean(dy)) * rstd with xhat = xc * rstd (xc = x - mean, what xv holds):
+            //    = dy * rstd - xc * (rstd^3 mean(xc dy)) - mean(dy) * rstd
+            const float inner = group_reduce<G>(si) * p.inv_d;  // mean(xc dy)
             const float mdy = group_reduce<G>(sg) * p.inv_d;
+            const float cx = -(rstd * rstd) * (rstd * inner), c0 = -mdy * rstd;
 #pragma unroll
             for (int k = 0; k < NV; ++k)
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) out[k][e] = (dv[k][e] - xv[k][e] * inner - mdy) * rstd;
+                for (int e = 0; e < VEC; ++e) out[k][e] = fmaf(xv[k][e], cx, fmaf(dv[k][e], rstd, c0));
         }
 #pragma unroll
-        for (int k = 0; k < NV; ++k) store_chunk<T, VEC, VECTOR, RGD_HEAD_NT_STORE != 0>(yrow[u], (k * G + lg) * VEC, lim[u], out[k]);
+        for (int k = 0; k < NV; ++k) {
+            if constexpr (COMPACT)
+                store_chunk_at<T, VEC, RGD_HEAD_NT_STORE != 0>(h.y, yoff[u] + k * (uint32_t)(G * VEC * sizeof(T)), lim[u] != 0, out[k]);
+            else
+                store_chunk<T, VEC, VECTOR, RGD_HEAD_NT_STORE != 0>(yrow[u], (k * G + lg) * VEC, lim[u], out[k]);
+        }
     }
     }  // row blocks of this workgroup
 }
@@ -200,6 +251,7 @@ struct HeadConfig {
     int mode;
     int G, NV;
     bool vector;
+    bool compact;    // rows at equal distances, 31-bit byte offsets (see head_rows_kernel)
     bool table_f32;  // rotary table is fp32 while the tensors are 16-bit
 };
 #ifndef RGD_HEAD_U_FWD

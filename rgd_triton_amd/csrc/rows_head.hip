@@ -120,6 +120,33 @@ int head_launch(const char* name, int mode, int64_t B, int64_t H, int64_t Tq, in
     }
 
     cfg.vector = vector;
+    // COMPACT addressing: every tensor's rows at one distance in iteration order, all byte offsets below 2^31
+    bool compact = vector;
+    const int64_t lim31 = (int64_t(1) << 31) - 64;
+    for (int i = 0; i < 2 && compact; ++i) {
+        HeadHalf& h = p.h[i];
+        if (h.rows == 0) continue;
+        const int64_t n2 = h.n2, n1 = h.n12 / h.n2;
+        auto distance = [&](const int64_t* st, uint32_t* out) {
+            const int64_t dist = n2 > 1 ? st[2] : (n1 > 1 ? st[1] : st[0]);
+            // (row index and row distance below 2^24 each: the kernel multiplies them with the 24-bit multiplier)
+            const bool ok = dist >= 0 && (n2 == 1 || st[2] == dist) && (n1 == 1 || st[1] == dist * n2) &&
+                            (B == 1 || st[0] == dist * n1 * n2) && ((int64_t)h.rows * dist + D) * es < lim31 &&
+                            h.rows < (1u << 24) && dist * es < (1 << 24);
+            *out = ok ? (uint32_t)(dist * es) : 0u;
+            return ok;
+        };
+        compact = distance(h.sx, &h.rbx) && distance(h.sy, &h.rby) && (!bwd || distance(h.sd, &h.rbd));
+    }
+    if (compact && rope) {
+        const int64_t ps = rope->R == 0 ? 1 : rgd_dtype_size(rope->dtype);
+        compact = p.pe_sn >= 0 && p.pe_ss >= 0 && rope->P < (1 << 24) && p.pe_sn * ps < (1 << 24) &&
+                  (rope->P * p.pe_sn + D) * ps < lim31 && p.pe_ss * ps < lim31 &&
+                  (rope->P * p.pe_sn + D) * ps + p.pe_ss * ps < lim31;
+        p.pe_row_bytes = (uint32_t)(p.pe_sn * ps);
+        p.pe_cos_bytes = (uint32_t)(p.pe_ss * ps);
+    }
+    cfg.compact = compact;
     const int vec = vector ? 16 / es : 2;
     const int chunks = (int)((D + vec - 1) / vec);
     if (chunks <= 64) {

@@ -4,19 +4,22 @@
 #include "rows_head.h"
 
 template <typename T, typename TP, int MODE, int G, int NV, bool VECTOR>
-static int head_launch_one(const HeadParams& p, dim3 grid, hipStream_t s) {
+static int head_launch_one(const HeadParams& p, bool compact, dim3 grid, hipStream_t s) {
     constexpr int VEC = VECTOR ? 16 / (int)sizeof(T) : 2;
     constexpr int U = head_unroll(MODE, NV);
     // rows that fill their lane group exactly (the power-of-two head dims) skip every range mask
-    if (VECTOR && p.D == G * NV * VEC)
+    if (VECTOR && p.D == G * NV * VEC) {
+        if (compact)
+            return rgd_launch_status("head rows", rgd_launch(head_rows_kernel<T, TP, MODE, G, NV, VEC, VECTOR, VECTOR, U, VECTOR>, grid, dim3(256), 0, s, p));
         return rgd_launch_status("head rows", rgd_launch(head_rows_kernel<T, TP, MODE, G, NV, VEC, VECTOR, VECTOR, U>, grid, dim3(256), 0, s, p));
+    }
     return rgd_launch_status("head rows", rgd_launch(head_rows_kernel<T, TP, MODE, G, NV, VEC, VECTOR, false, U>, grid, dim3(256), 0, s, p));
 }
 
 template <typename T, typename TP, int MODE, bool VECTOR>
 static int head_dispatch_shape(const HeadConfig& c, const HeadParams& p, dim3 grid, hipStream_t s) {
 #define HEAD_CASE(g, nv) \
-    if (c.G == g && c.NV == nv) return head_launch_one<T, TP, MODE, g, nv, VECTOR>(p, grid, s);
+    if (c.G == g && c.NV == nv) return head_launch_one<T, TP, MODE, g, nv, VECTOR>(p, c.compact, grid, s);
     HEAD_CASE(4, 1)
     HEAD_CASE(8, 1)
     HEAD_CASE(16, 1)
