@@ -33,8 +33,8 @@ struct HeadHalf {
 };
 
 #ifndef RGD_HEAD_PERSIST
-#define RGD_HEAD_PERSIST 16  // at most this many workgroups per compute unit, each walking several row blocks
-// (measured on q,k (8,2048,16,64) bf16: 16 per unit shortens the LN+RoPE backward by 3 %; 4 and 8 lengthen both kernels by 5 %)
+#define RGD_HEAD_PERSIST 32  // at most this many workgroups per compute unit, each walking several row blocks
+// (measured on q,k (8,2048,16,64) bf16: 8 per unit lengthens the LN+RoPE step by 4 %, 16 by 1 %; 32, 64 and no cap are the same)
 #endif
 #ifndef RGD_HEAD_NT_STORE
 #define RGD_HEAD_NT_STORE 0

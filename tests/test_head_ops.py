@@ -54,6 +54,47 @@ def test_head_ln_layout_invariance_and_views():
     assert torch.equal(a_q, c_q)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads_second", [True, False])
+@pytest.mark.parametrize("which", ["ln", "rope", "ln_rope"])
+def test_head_ops_compact_addressing_equals_general(which, heads_second, dtype):
+    """Tensors whose rows lie at one distance (contiguous ones) take kernels that address them with a base and a 32-bit
+    offset; any other layout takes the general kernels.  The same values through both, forward and backward, must give
+    the same bits: here contiguous tensors against views into buffers with one spare head between the tokens."""
+    from rgd_triton_amd import triton_fused_ln_func_fn, triton_fused_ln_rope_fn, triton_rope_fn
+
+    g = gen(31)
+    B, H, Tq, Tk, D, R = 3, 5, 150, 97, 64, 32
+    q, k = _qk(g, B, H, Tq, Tk, D, dtype, heads_second, shift=0.3, scale=1.5)
+    gq, gk = _qk(g, B, H, Tq, Tk, D, dtype, heads_second)
+    pe = oracle.rotary_table(max(Tq, Tk) + 1, R, dtype=dtype).to("cuda")
+    cut = (Tq * 3 // 4, Tk)
+
+    def spread(t):
+        """the same values as a view with a spare head (heads_second: a spare token) between the rows of a token"""
+        t = t.cuda()
+        big = torch.full((t.shape[0], t.shape[1], t.shape[2] + 1, t.shape[3]), float("nan"), dtype=t.dtype, device="cuda")
+        view = big[:, :, : t.shape[2]]
+        view.copy_(t)
+        return view
+
+    def run(a, b, ga, gb):
+        a, b = a.detach().requires_grad_(True), b.detach().requires_grad_(True)
+        if which == "ln":
+            out = triton_fused_ln_func_fn(a, b, heads_second, 1e-6)
+        elif which == "rope":
+            out = triton_rope_fn(a, b, pe, cut, heads_second)
+        else:
+            out = triton_fused_ln_rope_fn(a, b, pe, cut, heads_second)
+        return (*out, *torch.autograd.grad(out, (a, b), (ga, gb)))
+
+    dense = run(q.cuda(), k.cuda(), gq.cuda(), gk.cuda())
+    spaced = run(spread(q), spread(k), spread(gq), spread(gk))
+    for a, b, n in zip(dense, spaced, ("qo", "ko", "dq", "dk")):
+        assert not torch.isnan(b.float()).any(), n
+        assert torch.equal(a, b), n
+
+
 # ---------------------------------------------------------------- RoPE
 def _table(P, R, dtype, axial=False):
     if axial:
