@@ -81,6 +81,31 @@ def test_error_paths_return_codes_without_a_gpu():
     assert lib.rgd_rms_bwd(4, 1024, 1024, t3, t3, t3, t3, t3, 1, 0, 0, 1e-6, 0x1000, 16, None) == -4
 
 
+def test_set_up_does_not_latch_without_a_device():
+    """Without a usable GPU rgd_init reports that and keeps nothing: the argument checks and workspace queries above still
+    work afterwards, and a second call says the same again.  (With a GPU it returns 0 and the test ends there.)"""
+    import torch
+
+    lib = _hip.lib()
+    rc = lib.rgd_init()
+    if torch.cuda.is_available():
+        assert rc == 0, lib.rgd_last_error()
+        return
+    assert rc == -3 and b"no usable device" in lib.rgd_last_error()
+    assert lib.rgd_attn_bwd_workspace(1, 2, 64, 64, 64, 1) > 0 and lib.rgd_rms_bwd_workspace(4, 1024, 1024, 0, 0) > 0
+    assert lib.rgd_init() == -3
+    # tile classes: sizes are plain host arithmetic
+    shared = _hip.Tensor4(0x1000, 64 * 128, 0, 128)
+    n = lib.rgd_attn_bias_classes_bytes(2, 4, 64, 128, 64, shared, _hip.BIAS_MATRIX, 2)
+    assert n > 0 and n % 8 == 0
+    assert lib.rgd_attn_bias_classes_bytes(2, 4, 64, 128, 128, shared, _hip.BIAS_MATRIX, 2) == 0       # head dim above 64
+    per_head = _hip.Tensor4(0x1000, 4 * 64 * 128, 64 * 128, 128)
+    assert lib.rgd_attn_bias_classes_bytes(2, 4, 64, 128, 64, per_head, _hip.BIAS_MATRIX, 2) == 0     # not shared by the heads
+    assert lib.rgd_attn_bias_classes_bytes(2, 4, 64, 128, 64, shared, _hip.BIAS_VECTOR, 2) == n       # a vector: the same map
+    assert lib.rgd_attn_bias_classify(2, 4, 64, 128, 64, shared, _hip.BIAS_MATRIX, 2, 0x1000, 8, None) == -4
+    assert b"classes" in lib.rgd_last_error()
+
+
 def test_module_api_surface_matches_reference():
     import rgd_triton_amd as rgd
 
