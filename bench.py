@@ -13,7 +13,7 @@ independent buffer sets (4 x 268 MB) are used in rotation so that no step finds 
 Prints ONE JSON line: value = algorithmic GB/s of the whole step, `roofline` for the dominant
 kernel (the backward) from HIP events recorded around every launch inside the timed region,
 (minus the measured cost of an event), `cpu_baseline` = the CPU oracle timed on this host on a bounded sample, and `extra` with the other
-BASELINE configurations (attention TFLOP/s, RMSNorm2 / head LayerNorm GB/s) and the Module-API timing.
+benchmark configurations (attention TFLOP/s, RMSNorm2 / head LayerNorm GB/s) and the Module-API timing.
 """
 import argparse
 import ctypes

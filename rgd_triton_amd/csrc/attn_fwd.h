@@ -597,7 +597,7 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
     // CLS: the class of the tile goes into the step as a scalar (read from LDS a step ahead)
     auto step = [&](const int j, auto FAST, auto AHEAD, auto WBIAS) __attribute__((always_inline)) {
         if constexpr (CLS) {
-#ifdef RGD_CLS_DEBUG_NOCHECK
+#ifdef RGD_CLS_DEBUG_NOCHECK  // timing-only build (wrong results unless every tile is ZERO): what the class test costs
             tile_step(j, FAST, AHEAD, IntC<0>{}, CLS_ZERO);
 #else
             const int tc = __builtin_amdgcn_readfirstlane(cls_ahead);

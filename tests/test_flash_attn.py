@@ -242,7 +242,7 @@ def test_flash_attn_bwd_transpose(Tq, Tk, dtype):
 
 
 def test_flash_attn_masked_bias_no_nan():
-    """-inf in the bias: block-causal mask (blocks of 128, as BASELINE config 4) and padded keys
+    """-inf in the bias: block-causal mask (blocks of 128, as benchmark configuration 4) and padded keys
     (as config 5).  dk/dv rows of fully masked keys are exactly zero; nothing is NaN."""
     g = gen(6)
     B, H, T, d = 2, 3, 384, 64

@@ -1,4 +1,4 @@
-"""The BASELINE configurations at their full sizes.  The CPU oracle finishes these only on slices, so each
+"""The benchmark configurations at their full sizes.  The CPU oracle finishes these only on slices, so each
 configuration is checked through (a) the oracle on a slice that the operator computes independently of the
 rest (rows of a row operator, query rows of attention), and (b) properties that hold at any size: batch /
 head permutation equivariance (bit-exact), key permutation invariance, V = const -> O = const, a constant

@@ -77,7 +77,7 @@ def test_fused_equals_single():
 
 
 def test_fused_rms_config5_and_module():
-    """BASELINE config 5a: image (2,4096,1536) + text (2,256,1536) bf16 through the Module."""
+    """Benchmark configuration 5a: image (2,4096,1536) + text (2,256,1536) bf16 through the Module."""
     from rgd_triton_amd import FusedRMSNorm2
 
     g = gen(1005)

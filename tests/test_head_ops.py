@@ -231,7 +231,7 @@ def test_ln_rope_equals_ln_then_rope_fp32():
 
 
 def test_ln_rope_config2_slice():
-    """BASELINE config 2 at reduced batch: q,k (2,2048,16,64) bf16, heads_second=False, eps 1e-5,
+    """Benchmark configuration 2 at reduced batch: q,k (2,2048,16,64) bf16, heads_second=False, eps 1e-5,
     R=32, theta 10000, cutoff (2048,2048), P = 2049."""
     from rgd_triton_amd import FusedLNRoPE
 

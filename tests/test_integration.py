@@ -1,6 +1,6 @@
 """The operators inside the callers the reference describes: the README's Attention block
 (README.md:36-60: qkv Linear -> unbind -> FusedHeadLayerNorm -> FlashAttention -> out_proj) and the
-MMDiT-style joint block of BASELINE config 5 (FusedRMSNorm2 on image+text streams -> projections ->
+MMDiT-style joint block of benchmark configuration 5 (FusedRMSNorm2 on image+text streams -> projections ->
 FusedHeadLayerNorm -> FlashAttention with a broadcast padding bias), forward and backward, against the
 same block built from the CPU oracle's math with PyTorch autograd."""
 import math
@@ -87,7 +87,7 @@ def test_readme_attention_block(with_bias, dtype):
 
 @pytest.mark.parametrize("size", ["reduced", "config5"])
 def test_mmdit_joint_block_chain(size):
-    """BASELINE config 5 as a chain (the [image || text] joint sequence, -inf bias on ~10 % of the text keys per batch
+    """benchmark configuration 5 as a chain (the [image || text] joint sequence, -inf bias on ~10 % of the text keys per batch
     element, everything bf16), at a reduced size and at its real size (2 x (4096 + 256) tokens, 1536 channels, 24 heads
     of 64), forward and backward against the same chain in fp32 PyTorch on the CPU."""
     from rgd_triton_amd import FlashAttention, FusedHeadLayerNorm, FusedRMSNorm2

@@ -88,7 +88,7 @@ def test_rms_mixed_weight_dtype(dtype, wdtype):
 
 
 def test_rms_config1_fp32_tight():
-    """BASELINE config 1: (4,1024,1024) fp32, w = 1 + 0.1 N(0,1), eps 1e-6; fp32 bar <= 1e-5 relative."""
+    """Benchmark configuration 1: (4,1024,1024) fp32, w = 1 + 0.1 N(0,1), eps 1e-6; fp32 bar <= 1e-5 relative."""
     (y, dx, dw), (y_ref, dx_ref, dw_ref) = _run(4, 1024, 1024, torch.float32, False, seed=1001)
     for a, r, n in ((y, y_ref, "y"), (dx, dx_ref, "dx"), (dw, dw_ref, "dw")):
         err = (a.cpu() - r).abs().max() / r.abs().max()
