@@ -12,6 +12,8 @@
 // independent of scheduling.  (Combining the rows inside the first kernel, with arrival tickets, was
 // measured slower: every level of such a tree costs several microseconds of cross-XCD round trips.)
 #pragma once
+
+#include <type_traits>
 #ifndef RGD_WIDE_RMS_FWD_64
 #define RGD_WIDE_RMS_FWD_64 1
 #endif
@@ -83,15 +85,31 @@ __global__ __launch_bounds__(NW * 64) void wide_rows_kernel(const WideParams p) 
     float dwacc[NV][VEC];
     if constexpr (HAS_W) {
         const char* wp = static_cast<const char*>(h.w) + (int64_t)b * h.sw_b * (h.w_dtype == RGD_F32 ? 4 : 2);
+        // The weight's element type and alignment are known at run time only.  One decision for the whole row, and inside
+        // it all NV chunk loads go out before the first is decoded: one round trip to memory in front of the row loop
+        // instead of NV of them (a kernel of the small configurations lasts a handful of such round trips).
+        auto load_w = [&](auto tag, auto vec_ok) __attribute__((always_inline)) {
+            typedef decltype(tag) TW;
+            constexpr bool V = decltype(vec_ok)::value;
+            Chunk<TW, VEC, V> wc[NV];
 #pragma unroll
-        for (int k = 0; k < NV; ++k) {
-            if (VECTOR && h.w_vec)
-                load_chunk_dyn<VEC, VECTOR>(wp, h.w_dtype, (k * GL + lg) * VEC, C, wv[k]);
-            else
-                load_chunk_dyn<VEC, false>(wp, h.w_dtype, (k * GL + lg) * VEC, C, wv[k]);
+            for (int k = 0; k < NV; ++k) wc[k].load(reinterpret_cast<const TW*>(wp), (k * GL + lg) * VEC, C);
+#pragma unroll
+            for (int k = 0; k < NV; ++k) wc[k].template decode<true>((k * GL + lg) * VEC, C, wv[k]);
+        };
+        if (VECTOR && h.w_vec) {
+            if (h.w_dtype == RGD_BF16) load_w(bf16_t{}, std::integral_constant<bool, VECTOR>{});
+            else if (h.w_dtype == RGD_F16) load_w(f16_t{}, std::integral_constant<bool, VECTOR>{});
+            else load_w(float{}, std::integral_constant<bool, VECTOR>{});
+        } else {
+            if (h.w_dtype == RGD_BF16) load_w(bf16_t{}, std::false_type{});
+            else if (h.w_dtype == RGD_F16) load_w(f16_t{}, std::false_type{});
+            else load_w(float{}, std::false_type{});
+        }
+#pragma unroll
+        for (int k = 0; k < NV; ++k)
 #pragma unroll
             for (int e = 0; e < VEC; ++e) dwacc[k][e] = 0.f;
-        }
     }
 
     // the trip count is the same for every wavefront of the block (rows past the end are masked), so the
