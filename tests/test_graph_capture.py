@@ -31,6 +31,10 @@ class _Sequence:
                         w1=(1 + 0.1 * torch.randn(384, generator=g)).to(dt).cuda(),
                         w2=(1 + 0.1 * torch.randn(640, generator=g)).to(dt).cuda(),
                         bias=(0.3 * torch.randn(B, 1, T, T, generator=g)).to(dt).cuda())
+        # the bias is shared by the heads, so the calls classify its tiles (inside the graph, when captured): batch
+        # element 0 is a key mask, served by the kernels that read the classes; element 1 is dense, served by the others
+        self.inp["bias"][0] = 0
+        self.inp["bias"][0, :, :, T - 90::3] = float("-inf")
         self.pe = oracle.rotary_table(T + 1, 32, 10000.0, dt).cuda()
         lib = self.lib
         self.rms_ws = torch.empty(max(lib.rgd_rms_bwd_workspace(B, T, 384, 77, 640), 1), dtype=torch.uint8, device="cuda")
@@ -88,6 +92,7 @@ def test_c_abi_sequence_replays_from_a_graph():
             t.fill_(float("nan"))
         for name in ("q", "x1", "v", "d2"):  # new values in the graph's input buffers (eager kernels)
             seq.inp[name].mul_(-0.75 if rep % 2 else 1.25)
+        seq.inp["bias"].copy_(seq.inp["bias"].flip(0))  # mask and dense bias change places: other classes on replay
         torch.cuda.synchronize()
         seq.run(eager_out)
         torch.cuda.synchronize()
