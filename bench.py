@@ -555,6 +555,58 @@ def head_ln_case(torch, name, B, T, H, D, dtype, nsets, with_cpu=False):
     return r
 
 
+def rope_case(torch, name, B, T, H, D, R, dtype, nsets):
+    """RoPE alone (rgd_rope_qk forward, then with the rotation sign flipped: its backward) on q and k"""
+    import rgd_oracle as oracle
+    from rgd_triton_amd import _hip
+
+    lib = _hip.lib()
+    code = _hip.dtype_code(dtype)
+    st = _hip.stream_ptr(torch.device("cuda"))
+    pe = oracle.rotary_table(T + 1, R, 10000.0, dtype).cuda()
+    pe_args = (ctypes.c_void_p(pe.data_ptr()), pe.shape[1], pe.shape[2], pe.stride(0), pe.stride(1), code)
+    mk = lambda: [torch.randn(B, T, H, D, device="cuda").to(dtype) for _ in range(nsets)]
+    q, k, gq, gk = mk(), mk(), mk(), mk()
+    qo, ko = [torch.empty_like(t) for t in q], [torch.empty_like(t) for t in k]
+    d = [{n: _hip.t4(x[i], False) for n, x in dict(q=q, k=k, gq=gq, gk=gk, qo=qo, ko=ko).items()} for i in range(nsets)]
+
+    def fwd(i):
+        assert lib.rgd_rope_qk(B, H, T, T, D, d[i]["q"], d[i]["k"], d[i]["qo"], d[i]["ko"], *pe_args, T, T, 0, code, st) == 0, \
+            lib.rgd_last_error()
+
+    def bwd(i):
+        assert lib.rgd_rope_qk(B, H, T, T, D, d[i]["gq"], d[i]["gk"], d[i]["qo"], d[i]["ko"], *pe_args, T, T, 1, code, st) == 0, \
+            lib.rgd_last_error()
+
+    n = 2 * B * T * H * D * torch.empty(0, dtype=dtype).element_size()
+    return rows_result(torch, name, fwd, bwd, 2 * n, 2 * n, nsets)  # the backward reads dy and writes dx: two passes
+
+
+def l2_case(torch, name, B, shapes, dtype, nsets):
+    """FusedL2Normalize2 forward+backward through the C ABI"""
+    from rgd_triton_amd import _hip
+
+    lib, t3 = _hip.lib(), _hip.t3
+    code = _hip.dtype_code(dtype)
+    es = torch.empty(0, dtype=dtype).element_size()
+    st = _hip.stream_ptr(torch.device("cuda"))
+    (T1, C1), (T2, C2) = shapes
+    mk = lambda T, C: [torch.randn(B, T, C, device="cuda").to(dtype) for _ in range(nsets)]
+    x1, d1, x2, d2 = mk(T1, C1), mk(T1, C1), mk(T2, C2), mk(T2, C2)
+    y1, y2 = [torch.empty_like(t) for t in x1], [torch.empty_like(t) for t in x2]
+
+    def fwd(i):
+        assert lib.rgd_fused_l2_fwd(B, T1, C1, T2, C2, t3(x1[i]), t3(y1[i]), t3(x2[i]), t3(y2[i]), code, 1e-6, st) == 0, \
+            lib.rgd_last_error()
+
+    def bwd(i):
+        assert lib.rgd_fused_l2_bwd(B, T1, C1, T2, C2, t3(d1[i]), t3(x1[i]), t3(y1[i]), t3(d2[i]), t3(x2[i]), t3(y2[i]), code, 1e-6,
+                                    st) == 0, lib.rgd_last_error()
+
+    n = B * (T1 * C1 + T2 * C2) * es
+    return rows_result(torch, name, fwd, bwd, 2 * n, 3 * n, nsets)
+
+
 def extras(torch, only="", with_cpu=False):
     import rgd_triton_amd as rgd
 
@@ -599,6 +651,10 @@ def extras(torch, only="", with_cpu=False):
                             [(4096, 1536), (256, 1536)], bf, 12, with_cpu=with_cpu))
     if want("rms_wide"):
         out.append(rms_case(torch, "rms_wide: FusedRMSNorm (8,4096,4096) bf16 fwd+bwd", 8, [(4096, 4096)], bf, 3, with_api=False))
+    if want("rope_c2"):
+        out.append(rope_case(torch, "rope_c2: RoPE q,k (8,2048,16,64) bf16, R=32, forward + backward rotation", 8, 2048, 16, 64, 32, bf, 4))
+    if want("l2x2_c5"):
+        out.append(l2_case(torch, "l2x2_c5: FusedL2Normalize2 (2,4096,1536)+(2,256,1536) bf16 fwd+bwd", 2, [(4096, 1536), (256, 1536)], bf, 12))
     if want("headln_c5"):
         out.append(head_ln_case(torch, "headln_c5: FusedHeadLayerNorm q,k (2,4352,24,64) bf16 fwd+bwd", 2, 4352, 24, 64, bf, 6, with_cpu=with_cpu))
     return out
