@@ -569,7 +569,7 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
     auto step = [&](const int j, auto FAST, auto AHEAD, auto WBIAS) __attribute__((always_inline)) {
         if constexpr (CLS) {
             const int tc = __builtin_amdgcn_readfirstlane(cls_ahead);
-            cls_ahead = cls_lds[min(j + 1, CLS_LDS_BYTES - 1)];
+            cls_ahead = cls_lds[min(j + 1, CLS_MAX_TILES - 1)];
             tile_step(j, FAST, AHEAD, IntC<0>{}, tc);
         } else {
             tile_step(j, FAST, AHEAD, WBIAS, 0);
@@ -613,16 +613,11 @@ __global__ __launch_bounds__(BWD_THREADS, (DPAD <= 64 || DqSmem<DPAD>::BN == 32)
     if constexpr (CLS) {
         // Runs of tiles that are not NEG go through the loop (the loop of the kernel without bias, plus the addition of the
         // bias on MIXED tiles); NEG runs (P = 0 and dS = 0) are left out, K/V loads and all.
-        int j = t_begin;
+        int j = cls_next_tile(cls_lds, t_begin, t_end, false);
         while (j < t_end) {
-            if (cls_lds_at(cls_lds, j) == CLS_NEG) {
-                ++j;
-                continue;
-            }
-            int e = j + 1;
-            while (e < t_end && cls_lds_at(cls_lds, e) != CLS_NEG) ++e;
+            const int e = cls_next_tile(cls_lds, j + 1, t_end, true);
             run_tiles(j, e, IntC<0>{});
-            j = e;
+            j = cls_next_tile(cls_lds, e, t_end, false);
         }
     } else {
         run_tiles(t_begin, t_end, IntC<(HAS_BIAS ? 1 : 0)>{});

@@ -67,25 +67,50 @@ inline BiasClasses cls_layout(const void* buffer, int64_t nb, int64_t Tq, int64_
     return c;
 }
 
-constexpr int CLS_LDS_BYTES = 2048;  // forward and dQ kernel: one byte per key tile
+constexpr int CLS_MAX_TILES = CLS_MAX_WORDS * CLS_TILES_PER_WORD;  // 2048
+constexpr int CLS_NEG_WORDS = CLS_MAX_TILES / 64;
+// forward and dQ kernel: one byte per key tile, then one bit per key tile (set: the tile is NEG)
+constexpr int CLS_LDS_BYTES = CLS_MAX_TILES + CLS_NEG_WORDS * 8;
 
 // Forward and dQ kernel: the class of every key tile for the workgroup's `nrows` rows of the map (its 128 query rows),
-// one byte per tile in LDS: ZERO / NEG when the tile is that in every one of the rows, MIXED otherwise.  What the
-// workgroup does with a tile (which loop runs it, whether its K/V are loaded at all) is then decided alike in all its
-// wavefronts, and nothing of the classes lives in registers while the loops run.  Ends with a barrier.
+// one byte per tile in LDS: ZERO / NEG when the tile is that in every one of the rows, MIXED otherwise; behind the bytes,
+// the NEG tiles as a bit mask (64 tiles per word), in which the loop driver finds the runs of tiles to work on with a
+// few scalar instructions per run instead of one LDS round trip per tile.  What the workgroup does with a tile (which
+// arm runs it, whether its K/V are loaded at all) is then decided alike in all its wavefronts, and nothing of the classes
+// lives in registers while the loops run.  256 threads; ends with a barrier.
 __device__ __forceinline__ void cls_tiles_to_lds(const BiasClasses& c, int b, int row0, int nrows, int ntiles, uint8_t* lds, int tid) {
-    for (int t = tid; t < ntiles; t += 256) {
+    uint64_t* neg_mask = reinterpret_cast<uint64_t*>(lds + CLS_MAX_TILES);
+    for (int base = 0; base < ntiles; base += 256) {  // (the same trip count in every wavefront: the ballot below)
+        const int t = base + tid;
         bool zero = true, neg = true, col = true;
-        for (int r = 0; r < nrows; ++r) {
-            const uint64_t w = c.words[b * c.sb + (int64_t)min(row0 + r, c.nrow32 - 1) * c.nwords + (t >> 5)];
-            const uint32_t f = (uint32_t)(w >> (2 * (t & 31))) & 3u;
-            zero = zero && f == CLS_ZERO;
-            neg = neg && f == CLS_NEG;
-            col = col && f != CLS_MIXED;  // each wavefront reads the first of its own 32 rows
+        if (t < ntiles) {
+            for (int r = 0; r < nrows; ++r) {
+                const uint64_t w = c.words[b * c.sb + (int64_t)min(row0 + r, c.nrow32 - 1) * c.nwords + (t >> 5)];
+                const uint32_t f = (uint32_t)(w >> (2 * (t & 31))) & 3u;
+                zero = zero && f == CLS_ZERO;
+                neg = neg && f == CLS_NEG;
+                col = col && f != CLS_MIXED;  // each wavefront reads the first of its own 32 rows
+            }
+            lds[t] = zero ? CLS_ZERO : (neg ? CLS_NEG : (col ? CLS_COLUMN : CLS_MIXED));
         }
-        lds[t] = zero ? CLS_ZERO : (neg ? CLS_NEG : (col ? CLS_COLUMN : CLS_MIXED));
+        const uint64_t m = __builtin_amdgcn_ballot_w64(t < ntiles && neg);
+        if ((tid & 63) == 0) neg_mask[t >> 6] = m;
     }
     __syncthreads();
+}
+// the first tile in [j, end) whose NEG bit equals `neg` (end if there is none); wavefront-uniform
+__device__ __forceinline__ int cls_next_tile(const uint8_t* lds, int j, int end, bool neg) {
+    const uint64_t* neg_mask = reinterpret_cast<const uint64_t*>(lds + CLS_MAX_TILES);
+    while (j < end) {
+        const uint64_t raw = neg_mask[j >> 6];
+        uint64_t w = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(raw >> 32)) << 32) |
+                     (uint32_t)__builtin_amdgcn_readfirstlane((int)raw);
+        if (!neg) w = ~w;
+        w &= ~0ull << (j & 63);
+        if (w != 0) return min(end, (j & ~63) + (int)__builtin_ctzll(w));
+        j = (j & ~63) + 64;
+    }
+    return end;
 }
 // class of tile / step j, the same value in every lane (a scalar for the compiler)
 __device__ __forceinline__ int cls_lds_at(const uint8_t* lds, int j) { return __builtin_amdgcn_readfirstlane((int)lds[j]); }

@@ -601,7 +601,7 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
             tile_step(j, FAST, AHEAD, IntC<0>{}, CLS_ZERO);
 #else
             const int tc = __builtin_amdgcn_readfirstlane(cls_ahead);
-            cls_ahead = cls_lds[min(j + 1, CLS_LDS_BYTES - 1)];
+            cls_ahead = cls_lds[min(j + 1, CLS_MAX_TILES - 1)];
             tile_step(j, FAST, AHEAD, IntC<0>{}, tc);
 #endif
         } else {
@@ -646,16 +646,11 @@ __global__ __launch_bounds__(ATTN_THREADS, CLS ? RGD_CLS_FWD_OCC : ((DPAD <= 64 
     if constexpr (CLS) {
         // Runs of tiles that are not NEG go through the loop (the loop of the kernel without bias, plus the addition of the
         // bias on MIXED tiles); NEG runs (every probability 0) are left out, K/V loads and all.
-        int j = t_begin;
+        int j = cls_next_tile(cls_lds, t_begin, t_end, false);
         while (j < t_end) {
-            if (cls_lds_at(cls_lds, j) == CLS_NEG) {
-                ++j;
-                continue;
-            }
-            int e = j + 1;
-            while (e < t_end && cls_lds_at(cls_lds, e) != CLS_NEG) ++e;
+            const int e = cls_next_tile(cls_lds, j + 1, t_end, true);
             run_tiles(j, e, IntC<0>{});
-            j = e;
+            j = cls_next_tile(cls_lds, e, t_end, false);
         }
     } else {
         run_tiles(t_begin, t_end, IntC<(HAS_BIAS ? 1 : 0)>{});
