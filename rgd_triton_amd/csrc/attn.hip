@@ -83,8 +83,8 @@ bool cls_eligible(int64_t H, int64_t Tq, int64_t Tk, int64_t D, const rgd_tensor
     return cls_nwords(Tk) <= CLS_MAX_WORDS && cls_nrow32(Tq) <= CLS_MAX_ROWS;
 }
 int64_t cls_batches(int64_t B, const rgd_tensor4* bias) { return bias->stride_b == 0 ? 1 : B; }
-BiasClasses cls_desc(const void* buffer, int64_t B, int64_t Tq, int64_t Tk, const rgd_tensor4* bias) {
-    return cls_layout(buffer, cls_batches(B, bias), Tq, Tk);
+BiasClasses cls_desc(const void* buffer, int64_t B, int64_t Tq, int64_t Tk, const rgd_tensor4* bias, int bias_kind) {
+    return cls_layout(buffer, cls_batches(B, bias), Tq, Tk, cls_row_stride(bias, bias_kind) == 0);
 }
 // The classes a call works with: the caller's (bias_classes), or written here into the end of the workspace when it has
 // room for them behind `fixed_bytes`; *room is what is left of the workspace in front of them.  Null: none.
@@ -225,7 +225,7 @@ int rgd_attn_fwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
                                                          workspace_bytes, 0, &part_room, s, &rc)
                                           : nullptr;
     if (rc != RGD_OK) return rc;
-    if (cls) p.cls = cls_desc(cls, B, Tq, Tk, bias);
+    if (cls) p.cls = cls_desc(cls, B, Tq, Tk, bias, bias_kind);
     // items of the last, partly filled round are split along the keys when a workspace is given
     const int dpad = attn_dpad(D);
     AttnSplit plan;
@@ -382,7 +382,7 @@ int rgd_attn_bwd(int64_t B, int64_t H, int64_t Tq, int64_t Tk, int64_t D, const 
         p.bias_vec = rgd_aligned16(bias->ptr) && (p.bias.sb % per16) == 0 && (p.bias.sh % per16) == 0 &&
                      (p.bias.sn % per16) == 0;
     }
-    if (cls) p.cls = cls_desc(cls, B, Tq, Tk, bias);
+    if (cls) p.cls = cls_desc(cls, B, Tq, Tk, bias, bias_kind);
     if (one_pass) {
         p.dq_accum = reinterpret_cast<float*>(static_cast<char*>(workspace) + delta_bytes);
         if (Tq > 0) {  // delta, and dq_accum = 0

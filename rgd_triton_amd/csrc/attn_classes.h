@@ -56,11 +56,13 @@ inline size_t cls_bytes(int64_t nb, int64_t Tq, int64_t Tk) {
 }
 
 // host: the parts of a classes buffer written for nb batch elements (nb = 1: one map that every batch element uses)
-inline BiasClasses cls_layout(const void* buffer, int64_t nb, int64_t Tq, int64_t Tk) {
+// one_row: every row of the bias is the same row (row stride 0: a vector, or a matrix expanded from one); the map then
+// has one row per batch element, which stands for all of them (the kernels clamp the row index to nrow32 - 1)
+inline BiasClasses cls_layout(const void* buffer, int64_t nb, int64_t Tq, int64_t Tk, bool one_row) {
     BiasClasses c;
     c.words = static_cast<const uint64_t*>(buffer);
     c.nwords = cls_nwords(Tk);
-    c.nrow32 = cls_nrow32(Tq);
+    c.nrow32 = one_row ? 1 : cls_nrow32(Tq);
     c.sb = nb == 1 ? 0 : (int64_t)c.nrow32 * c.nwords;
     c.info = reinterpret_cast<const uint32_t*>(static_cast<const char*>(buffer) + cls_words_bytes(nb, Tq, Tk));
     c.info_sb = nb == 1 ? 0 : cls_info_words(Tk);

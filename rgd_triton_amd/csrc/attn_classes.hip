@@ -3,7 +3,8 @@
 
 template <typename TB>
 static hipError_t classify_launch(const void* bias, int64_t sb, int64_t sn, int nb, int Tq, int Tk, uint64_t* words, hipStream_t s) {
-    const int nrow32 = cls_nrow32(Tq), nstrips = cls_nwords(Tk) * 4;
+    BiasClasses c = cls_layout(words, nb, Tq, Tk, sn == 0);
+    const int nrow32 = c.nrow32, nstrips = cls_nwords(Tk) * 4;
     const unsigned gx = (unsigned)(((int64_t)nrow32 * nstrips + 3) / 4);
     void (*kern)(const TB*, int64_t, int64_t, int, int, int, int, uint16_t*) = attn_bias_classify_kernel<TB>;
     const TB* bp = static_cast<const TB*>(bias);
@@ -12,7 +13,6 @@ static hipError_t classify_launch(const void* bias, int64_t sb, int64_t sn, int 
     hipError_t e = hipLaunchKernel(reinterpret_cast<const void*>(kern), dim3(gx, (unsigned)nb), dim3(256), args, 0, s);
     if (e != hipSuccess) return e;
     // the summaries behind the map, from the map and the bias
-    BiasClasses c = cls_layout(words, nb, Tq, Tk);
     uint32_t* info = const_cast<uint32_t*>(c.info);
     void (*sum)(const TB*, int64_t, int64_t, int, int, BiasClasses, uint32_t*) = attn_bias_summary_kernel<TB>;
     void* sargs[] = {&bp, &sb, &sn, &Tq, &Tk, &c, &info};
